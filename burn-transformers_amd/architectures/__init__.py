@@ -1,3 +1,3 @@
-"""Importing this package registers the architectures the library ships (GPT-2)."""
+"""Importing this package registers the architectures the library ships (GPT-2, Salopel)."""
 
-from . import gpt2  # noqa: F401
+from . import gpt2, salopel  # noqa: F401

@@ -1,6 +1,7 @@
 from .base import ConfigError, UnsupportedArchitecture, read_config_json
 from .gpt2 import GPT2Config
+from .salopel import SalopelConfig
 from .registry import Family, register_family, resolve_family, supported_names, unregister_family
 
-__all__ = ["ConfigError", "UnsupportedArchitecture", "read_config_json", "GPT2Config", "Family",
+__all__ = ["ConfigError", "UnsupportedArchitecture", "read_config_json", "GPT2Config", "SalopelConfig", "Family",
            "register_family", "resolve_family", "supported_names", "unregister_family"]

@@ -52,12 +52,15 @@ def supported_names():
 
 
 def resolve_family(config_json):
-    """The family a parsed config.json asks for: ``architectures[0]`` first, then ``model_type``."""
+    """The family a parsed config.json asks for: ``architectures[0]`` first, then ``architecture``,
+    then ``model_type``."""
     data = unwrap_text_config(config_json)
     candidates = []
     architectures = data.get("architectures")
     if isinstance(architectures, (list, tuple)):
         candidates += [a for a in architectures if isinstance(a, str)]
+    if isinstance(data.get("architecture"), str):      # some configurations name one architecture, as a string
+        candidates.append(data["architecture"])
     if isinstance(data.get("model_type"), str):
         candidates.append(data["model_type"])
     for name in candidates:

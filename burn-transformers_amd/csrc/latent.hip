@@ -1,0 +1,168 @@
+// Kernels of the latent attention mixer (queries and keys/values through normalised low-rank
+// latents; only the key/value latent is cached, and attention runs on it directly).
+//   * latent norms: the two RMS norms behind the fused down-projection; the query latent goes to a
+//     buffer for the next product, the key/value latent straight into the paged cache, where it is
+//     the one shared "head" whose keys and values are the same vector
+//   * head projection with gate: per head out = sigmoid(g) * (W_h . ctx_h), the value up-projection
+//     applied AFTER the weighted sum over positions (it is linear, so it commutes with the sum)
+// Statistics and sums are 32-bit.
+#include "host.h"
+
+struct LatentNormCall {
+  int dtype;              // element type of `q_out` and of the cache: 0 float32, 1 bfloat16
+  int tokens;
+  int q_rank, q_cols;     // the query latent's length; columns of q_out written (latent, then zeros)
+  int kv_rank;            // the key/value latent's length (the cache's head size may be larger: zeros)
+  int kv_offset;          // its first column in `in`
+  float eps;
+  const float* in;        // [tokens][ld] float32: the fused down-projection
+  int64_t ld;
+  const float* q_gamma;   // [q_rank]
+  const float* kv_gamma;  // [kv_rank]
+  void* q_out;            // [tokens][ld_q]
+  int64_t ld_q;
+  const int* tok_seq;
+  const int* tok_pos;
+  KvView kv;              // one head of head_dim >= kv_rank
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) latent_norm_kernel(LatentNormCall c) {
+  __shared__ float scratch[32];
+  const int t = blockIdx.x;
+  const bool query = blockIdx.y == 0;
+  const int n = query ? c.q_rank : c.kv_rank;
+  const float* row = c.in + (int64_t)t * c.ld + (query ? 0 : c.kv_offset);
+  const float* gamma = query ? c.q_gamma : c.kv_gamma;
+  float partial = 0.f;
+  for (int col = threadIdx.x; col < n; col += blockDim.x) partial += row[col] * row[col];
+  const float rstd = 1.0f / sqrtf(block_sum(partial, scratch) / (float)n + c.eps);
+  if (query) {
+    T* out = static_cast<T*>(c.q_out) + (int64_t)t * c.ld_q;
+    for (int col = threadIdx.x; col < c.q_cols; col += blockDim.x)
+      out[col] = from_float<T>(col < n ? row[col] * rstd * gamma[col] : 0.f);
+  } else {
+    const int seq = c.tok_seq[t], pos = c.tok_pos[t], hd = c.kv.head_dim;
+    const int64_t base = kv_block_base(c.kv, seq, pos, 0);
+    T* keys = static_cast<T*>(c.kv.keys) + base;
+    T* values = static_cast<T*>(c.kv.values) + base;
+    for (int col = threadIdx.x; col < hd; col += blockDim.x) {
+      const T v = from_float<T>(col < n ? row[col] * rstd * gamma[col] : 0.f);
+      keys[key_offset(hd, pos, col)] = v;
+      values[value_offset(hd, pos, col)] = v;
+    }
+  }
+}
+
+BT_EXPORT int bt_latent_norm_call(void* stream, const LatentNormCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->q_rank <= 0 || c->kv_rank <= 0) BT_REFUSE("latent_norm: ranks %d and %d must be positive", c->q_rank, c->kv_rank);
+  if (c->kv.kv_heads != 1 || c->kv.head_dim < c->kv_rank)
+    BT_REFUSE("latent_norm: the cache keeps %d heads of %d, expected one of at least %d", c->kv.kv_heads,
+              c->kv.head_dim, c->kv_rank);
+  if (c->q_cols < c->q_rank || c->ld_q < c->q_cols || c->ld < c->kv_offset + c->kv_rank || c->kv_offset < c->q_rank)
+    BT_REFUSE("latent_norm: the rows do not hold the latents");
+  if (!c->in || !c->q_gamma || !c->kv_gamma || !c->q_out || !c->tok_seq || !c->tok_pos || !c->kv.blocks ||
+      !c->kv.keys || !c->kv.values)
+    BT_REFUSE("latent_norm: missing operand");
+  dim3 grid(c->tokens, 2), block(256);
+  if (c->dtype == 0)
+    hipLaunchKernelGGL(latent_norm_kernel<float>, grid, block, 0, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(latent_norm_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, *c);
+  return bt_check_launch("latent_norm");
+}
+
+// out[t][h * vdim + v] = sigmoid(gate[t][h * vdim + v]) * sum_r W[h * vdim + v][r] * ctx[t][h * ld_head + r]
+// One work-group per (tile of HP_TOKENS tokens, head, run of up to HP_VCHUNK outputs); the rank is
+// walked in steps of HP_RSTEP through LDS (the weights transposed, so that threads with consecutive
+// outputs read consecutive words).
+#define HP_TOKENS 16
+#define HP_VCHUNK 128
+#define HP_RSTEP 32
+#define HP_PER_THREAD (HP_TOKENS * HP_VCHUNK / 256)
+
+struct HeadProjectCall {
+  int dtype;              // element type of ctx, W and out
+  int tokens;
+  int heads, vdim, rank;
+  int head_pitch;         // elements between two heads' vectors in a row of ctx
+  int out_cols;           // columns of out written: heads * vdim, then zeros
+  const void* ctx;        // [tokens][ld_ctx]
+  int64_t ld_ctx;
+  const void* W;          // [heads * vdim][rank]
+  const float* gate;      // [tokens][ld_gate] pre-activation, or null
+  int64_t ld_gate;
+  void* out;              // [tokens][ld_out]
+  int64_t ld_out;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) head_project_kernel(HeadProjectCall c) {
+  __shared__ float ws[HP_RSTEP][HP_VCHUNK + 1];
+  __shared__ float cs[HP_TOKENS][HP_RSTEP + 1];
+  const int t0 = blockIdx.x * HP_TOKENS, head = blockIdx.y, v0 = blockIdx.z * HP_VCHUNK;
+  const int vc = min(HP_VCHUNK, c.vdim - v0);
+  const T* ctx = static_cast<const T*>(c.ctx);
+  const T* W = static_cast<const T*>(c.W) + ((int64_t)head * c.vdim + v0) * c.rank;
+  float acc[HP_PER_THREAD];
+#pragma unroll
+  for (int k = 0; k < HP_PER_THREAD; ++k) acc[k] = 0.f;
+  for (int r0 = 0; r0 < c.rank; r0 += HP_RSTEP) {
+    for (int e = threadIdx.x; e < HP_VCHUNK * HP_RSTEP; e += 256) {
+      const int v = e / HP_RSTEP, rr = e % HP_RSTEP;
+      ws[rr][v] = (v < vc && r0 + rr < c.rank) ? to_float(W[(int64_t)v * c.rank + r0 + rr]) : 0.f;
+    }
+    for (int e = threadIdx.x; e < HP_TOKENS * HP_RSTEP; e += 256) {
+      const int i = e / HP_RSTEP, rr = e % HP_RSTEP;
+      cs[i][rr] = (t0 + i < c.tokens && r0 + rr < c.rank)
+                      ? to_float(ctx[(int64_t)(t0 + i) * c.ld_ctx + (int64_t)head * c.head_pitch + r0 + rr]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < HP_PER_THREAD; ++k) {
+      const int e = threadIdx.x + 256 * k;
+      const int i = e / HP_VCHUNK, v = e % HP_VCHUNK;
+      float sum = acc[k];
+#pragma unroll
+      for (int rr = 0; rr < HP_RSTEP; ++rr) sum = fmaf(cs[i][rr], ws[rr][v], sum);
+      acc[k] = sum;
+    }
+    __syncthreads();
+  }
+  T* out = static_cast<T*>(c.out);
+#pragma unroll
+  for (int k = 0; k < HP_PER_THREAD; ++k) {
+    const int e = threadIdx.x + 256 * k;
+    const int i = e / HP_VCHUNK, v = e % HP_VCHUNK;
+    if (t0 + i >= c.tokens || v >= vc) continue;
+    const int col = head * c.vdim + v0 + v;
+    float y = acc[k];
+    if (c.gate) y *= 1.0f / (1.0f + expf(-c.gate[(int64_t)(t0 + i) * c.ld_gate + col]));
+    out[(int64_t)(t0 + i) * c.ld_out + col] = from_float<T>(y);
+  }
+  // the columns behind the last head's, which the next product reads as zeros
+  if (head == c.heads - 1 && blockIdx.z == gridDim.z - 1)
+    for (int e = threadIdx.x; e < HP_TOKENS * (c.out_cols - c.heads * c.vdim); e += 256) {
+      const int extra = c.out_cols - c.heads * c.vdim;
+      const int i = e / extra, col = c.heads * c.vdim + e % extra;
+      if (t0 + i < c.tokens) out[(int64_t)(t0 + i) * c.ld_out + col] = from_float<T>(0.f);
+    }
+}
+
+BT_EXPORT int bt_head_project_call(void* stream, const HeadProjectCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->heads <= 0 || c->vdim <= 0 || c->rank <= 0)
+    BT_REFUSE("head_project: %d heads of %d from rank %d: all must be positive", c->heads, c->vdim, c->rank);
+  if (c->head_pitch < c->rank || c->ld_ctx < (int64_t)c->heads * c->head_pitch ||
+      c->out_cols < c->heads * c->vdim || c->ld_out < c->out_cols ||
+      (c->gate && c->ld_gate < (int64_t)c->heads * c->vdim))
+    BT_REFUSE("head_project: the rows do not hold %d heads", c->heads);
+  if (!c->ctx || !c->W || !c->out) BT_REFUSE("head_project: missing operand");
+  dim3 grid((c->tokens + HP_TOKENS - 1) / HP_TOKENS, c->heads, (c->vdim + HP_VCHUNK - 1) / HP_VCHUNK), block(256);
+  if (c->dtype == 0)
+    hipLaunchKernelGGL(head_project_kernel<float>, grid, block, 0, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(head_project_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, *c);
+  return bt_check_launch("head_project");
+}

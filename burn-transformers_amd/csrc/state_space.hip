@@ -1,0 +1,429 @@
+// Kernels of the recurrent (state-space) mixers.  Everything that enters a recurrence is 32-bit:
+// step sizes, decays, states, the sums over the state.  A sequence's state lives in its slot's row
+// of the cache's per-sequence state area and is carried from step to step; a step may bring any
+// number of a sequence's tokens, which are walked in order.
+//   * causal convolution per channel with bias and silu; its last taps - 1 inputs are state
+//   * dt projection: softplus(W low + b)
+//   * selective scan (one state row per channel, one decay per state element), with the output gate
+//   * scan with one decay per head and a state of [state, head size] (state-space duality form)
+//   * gate, then RMS norm in equal parts
+#include "host.h"
+
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float softplus_f(float v) { return v > 20.0f ? v : log1pf(expf(v)); }
+
+// ---------------------------------------------------------------------------------------------
+struct CausalConvCall {
+  int cast_dtype;         // element type of `cast`
+  int tokens, n_seqs, channels, taps;
+  int cast_cols;          // columns of `cast` written: the channels, then zeros
+  const float* in;        // [tokens][ld_in]
+  int64_t ld_in;
+  const float* weight;    // [channels][taps]; the last tap meets the current token
+  const float* bias;      // [channels]
+  float* out;             // [tokens][ld_out] float32
+  int64_t ld_out;
+  void* cast;             // [tokens][ld_cast] the same in the products' type, or null
+  int64_t ld_cast;
+  float* state;           // slot s: [taps - 1][channels] at state + s * state_stride, oldest first
+  int64_t state_stride;
+  const int* tok_seq;
+  const int* seq_off;     // [n_seqs + 1]
+  const int* slots;       // [n_seqs]
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) causal_conv_kernel(CausalConvCall c) {
+  const int t = blockIdx.x;
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  T* cast = static_cast<T*>(c.cast);
+  if (ch >= c.channels) {
+    if (cast && ch < c.cast_cols) cast[(int64_t)t * c.ld_cast + ch] = from_float<T>(0.f);
+    return;
+  }
+  const int seq = c.tok_seq[t];
+  const int local = t - c.seq_off[seq];
+  const float* held = c.state + (int64_t)c.slots[seq] * c.state_stride;
+  float sum = c.bias[ch];
+  for (int j = 0; j < c.taps; ++j) {
+    const int back = c.taps - 1 - j;
+    const int src = local - back;
+    const float u = src >= 0 ? c.in[(int64_t)(t - back) * c.ld_in + ch]
+                             : held[(int64_t)(c.taps - 1 + src) * c.channels + ch];
+    sum = fmaf(c.weight[(int64_t)ch * c.taps + j], u, sum);
+  }
+  const float y = silu_f(sum);
+  c.out[(int64_t)t * c.ld_out + ch] = y;
+  if (cast) cast[(int64_t)t * c.ld_cast + ch] = from_float<T>(y);
+}
+
+// After the convolution: the state becomes the last taps - 1 inputs of each sequence.
+__global__ void __launch_bounds__(256) conv_state_kernel(CausalConvCall c) {
+  const int seq = blockIdx.x;
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  if (ch >= c.channels) return;
+  const int first = c.seq_off[seq], count = c.seq_off[seq + 1] - first;
+  float* held = c.state + (int64_t)c.slots[seq] * c.state_stride;
+  for (int r = 0; r < c.taps - 1; ++r) {
+    const int src = count - (c.taps - 1) + r;
+    // (an older input moves up: row r + count lies behind row r, and is read before it is written)
+    held[(int64_t)r * c.channels + ch] = src >= 0 ? c.in[(int64_t)(first + src) * c.ld_in + ch]
+                                                  : held[(int64_t)(r + count) * c.channels + ch];
+  }
+}
+
+BT_EXPORT int bt_causal_conv_call(void* stream, const CausalConvCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->channels <= 0 || c->taps <= 0 || c->n_seqs <= 0)
+    BT_REFUSE("causal_conv: %d channels, %d taps, %d sequences: all must be positive", c->channels, c->taps, c->n_seqs);
+  if (!c->in || !c->weight || !c->bias || !c->out || !c->tok_seq || !c->seq_off || !c->slots || (c->taps > 1 && !c->state))
+    BT_REFUSE("causal_conv: missing operand");
+  if (c->ld_in < c->channels || c->ld_out < c->channels || (c->cast && (c->cast_cols < c->channels || c->ld_cast < c->cast_cols)))
+    BT_REFUSE("causal_conv: the rows do not hold %d channels", c->channels);
+  if (c->taps > 1 && c->state_stride < (int64_t)(c->taps - 1) * c->channels)
+    BT_REFUSE("causal_conv: a slot's state of %lld elements does not hold %d inputs of %d channels",
+              (long long)c->state_stride, c->taps - 1, c->channels);
+  const int cols = c->cast && c->cast_cols > c->channels ? c->cast_cols : c->channels;
+  dim3 grid(c->tokens, (cols + 255) / 256), block(256);
+  if (c->cast_dtype == 0)
+    hipLaunchKernelGGL(causal_conv_kernel<float>, grid, block, 0, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(causal_conv_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, *c);
+  int rc = bt_check_launch("causal_conv");
+  if (rc || c->taps == 1) return rc;
+  hipLaunchKernelGGL(conv_state_kernel, dim3(c->n_seqs, (c->channels + 255) / 256), block, 0, (hipStream_t)stream, *c);
+  return bt_check_launch("causal_conv state");
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t][c] = softplus(sum_r W[c][r] * low[t][r] + bias[c]); the rank is small.
+struct DtProjectCall {
+  int dtype;              // element type of W
+  int tokens, channels, rank;
+  const float* low;       // [tokens][ld_low]
+  int64_t ld_low;
+  const void* W;          // [channels][rank]
+  const float* bias;      // [channels]
+  float* out;             // [tokens][ld_out]
+  int64_t ld_out;
+};
+
+#define DT_TOKENS 8
+
+template <typename T>
+__global__ void __launch_bounds__(256) dt_project_kernel(DtProjectCall c) {
+  extern __shared__ float rows[];      // [DT_TOKENS][rank]
+  const int t0 = blockIdx.x * DT_TOKENS;
+  for (int e = threadIdx.x; e < DT_TOKENS * c.rank; e += blockDim.x) {
+    const int i = e / c.rank, r = e % c.rank;
+    rows[e] = t0 + i < c.tokens ? c.low[(int64_t)(t0 + i) * c.ld_low + r] : 0.f;
+  }
+  __syncthreads();
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  if (ch >= c.channels) return;
+  const T* w = static_cast<const T*>(c.W) + (int64_t)ch * c.rank;
+  float acc[DT_TOKENS];
+#pragma unroll
+  for (int i = 0; i < DT_TOKENS; ++i) acc[i] = 0.f;
+  for (int r = 0; r < c.rank; ++r) {
+    const float wv = to_float(w[r]);
+#pragma unroll
+    for (int i = 0; i < DT_TOKENS; ++i) acc[i] = fmaf(wv, rows[i * c.rank + r], acc[i]);
+  }
+  const float b = c.bias[ch];
+#pragma unroll
+  for (int i = 0; i < DT_TOKENS; ++i)
+    if (t0 + i < c.tokens) c.out[(int64_t)(t0 + i) * c.ld_out + ch] = softplus_f(acc[i] + b);
+}
+
+BT_EXPORT int bt_dt_project_call(void* stream, const DtProjectCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->channels <= 0 || c->rank <= 0 || c->rank > 1024)
+    BT_REFUSE("dt_project: %d channels from rank %d (1..1024)", c->channels, c->rank);
+  if (!c->low || !c->W || !c->bias || !c->out || c->ld_low < c->rank || c->ld_out < c->channels)
+    BT_REFUSE("dt_project: missing operand or rows too short");
+  dim3 grid((c->tokens + DT_TOKENS - 1) / DT_TOKENS, (c->channels + 255) / 256), block(256);
+  size_t lds = (size_t)DT_TOKENS * c->rank * sizeof(float);
+  if (c->dtype == 0)
+    hipLaunchKernelGGL(dt_project_kernel<float>, grid, block, lds, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(dt_project_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, *c);
+  return bt_check_launch("dt_project");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Selective scan.  Per channel c and state element n, token after token of a sequence:
+//   S[c][n] <- exp(dt_c * A[c][n]) * S[c][n] + dt_c * x_c * B_n,   A = -exp(A_log)
+//   y_c = sum_n S[c][n] * C_n + D_c * x_c;   out_c = y_c * silu(z_c)
+// One wave per (8 channels, sequence): eight lanes share a channel, lane j of them owns the state
+// elements j, j + 8, ... in registers (R of them); a token's inputs are asked for U tokens at a time,
+// so that their latency is paid once per U tokens and not once per token.
+struct SelectiveScanCall {
+  int out_dtype;
+  int tokens, n_seqs, channels, state;
+  int out_cols;           // columns of out written: the channels, then zeros
+  const float* x;         // [tokens][ld_x] after convolution and silu
+  int64_t ld_x;
+  const float* z;         // [tokens][ld_z] gate, pre-activation
+  int64_t ld_z;
+  const float* dt;        // [tokens][ld_dt] after softplus
+  int64_t ld_dt;
+  const float* B;         // [tokens][ld_bc]
+  const float* C;         // [tokens][ld_bc]
+  int64_t ld_bc;
+  const float* A_log;     // [channels][state]
+  const float* D;         // [channels]
+  void* out;              // [tokens][ld_out]
+  int64_t ld_out;
+  float* S;               // slot s: [channels][state] at S + s * state_stride
+  int64_t state_stride;
+  const int* seq_off;
+  const int* slots;
+};
+
+template <typename T, int R, int U>
+__global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c) {
+  const int lane = threadIdx.x, sub = lane & 7;
+  const int ch = blockIdx.x * 8 + (lane >> 3), seq = blockIdx.y;
+  const bool live = ch < c.channels;
+  const int chs = live ? ch : c.channels - 1;        // idle lanes read a valid channel and write nothing
+  const int first = c.seq_off[seq], last = c.seq_off[seq + 1];
+  float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + (int64_t)chs * c.state;
+  float A[R], S[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int n = sub + 8 * r;
+    A[r] = n < c.state ? -expf(c.A_log[(int64_t)chs * c.state + n]) : 0.f;
+    S[r] = n < c.state ? held[n] : 0.f;
+  }
+  const float Dc = c.D[chs];
+  T* out = static_cast<T*>(c.out);
+  for (int t0 = first; t0 < last; t0 += U) {
+    float dt[U], xv[U], zv[U], Bv[U][R], Cv[U][R];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int t = min(t0 + u, last - 1);
+      dt[u] = c.dt[(int64_t)t * c.ld_dt + chs];
+      xv[u] = c.x[(int64_t)t * c.ld_x + chs];
+      zv[u] = c.z[(int64_t)t * c.ld_z + chs];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int n = sub + 8 * r;
+        Bv[u][r] = n < c.state ? c.B[(int64_t)t * c.ld_bc + n] : 0.f;
+        Cv[u][r] = n < c.state ? c.C[(int64_t)t * c.ld_bc + n] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (t0 + u < last) {
+        const float dx = dt[u] * xv[u];
+        float acc = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r] = expf(dt[u] * A[r]) * S[r] + dx * Bv[u][r];
+          acc = fmaf(S[r], Cv[u][r], acc);
+        }
+        acc += __shfl_xor(acc, 4, 64);
+        acc += __shfl_xor(acc, 2, 64);
+        acc += __shfl_xor(acc, 1, 64);
+        if (live && sub == 0)
+          out[(int64_t)(t0 + u) * c.ld_out + ch] = from_float<T>((acc + Dc * xv[u]) * silu_f(zv[u]));
+      }
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = sub + 8 * r;
+      if (n < c.state) held[n] = S[r];
+    }
+  }
+  // the columns behind the last channel, which the next product reads as zeros
+  if (blockIdx.x == 0)
+    for (int t = first; t < last; ++t)
+      for (int col = c.channels + lane; col < c.out_cols; col += 64) out[(int64_t)t * c.ld_out + col] = from_float<T>(0.f);
+}
+
+template <typename T>
+static int launch_selective_scan(hipStream_t stream, const SelectiveScanCall& c) {
+  dim3 grid((c.channels + 7) / 8, c.n_seqs), block(64);
+  const int per = (c.state + 7) / 8;
+  if (per <= 1) hipLaunchKernelGGL((selective_scan_kernel<T, 1, 8>), grid, block, 0, stream, c);
+  else if (per <= 2) hipLaunchKernelGGL((selective_scan_kernel<T, 2, 8>), grid, block, 0, stream, c);
+  else if (per <= 4) hipLaunchKernelGGL((selective_scan_kernel<T, 4, 4>), grid, block, 0, stream, c);
+  else if (per <= 8) hipLaunchKernelGGL((selective_scan_kernel<T, 8, 2>), grid, block, 0, stream, c);
+  else if (per <= 16) hipLaunchKernelGGL((selective_scan_kernel<T, 16, 1>), grid, block, 0, stream, c);
+  else hipLaunchKernelGGL((selective_scan_kernel<T, 32, 1>), grid, block, 0, stream, c);
+  return bt_check_launch("selective_scan");
+}
+
+BT_EXPORT int bt_selective_scan_call(void* stream, const SelectiveScanCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->channels <= 0 || c->state <= 0 || c->state > 256 || c->n_seqs <= 0)
+    BT_REFUSE("selective_scan: %d channels with %d state elements (1..256), %d sequences", c->channels, c->state, c->n_seqs);
+  if (!c->x || !c->z || !c->dt || !c->B || !c->C || !c->A_log || !c->D || !c->out || !c->S || !c->seq_off || !c->slots)
+    BT_REFUSE("selective_scan: missing operand");
+  if (c->ld_x < c->channels || c->ld_z < c->channels || c->ld_dt < c->channels || c->ld_bc < c->state ||
+      c->out_cols < c->channels || c->ld_out < c->out_cols || c->state_stride < (int64_t)c->channels * c->state)
+    BT_REFUSE("selective_scan: rows or state too short for %d channels of %d", c->channels, c->state);
+  return c->out_dtype == 0 ? launch_selective_scan<float>((hipStream_t)stream, *c)
+                           : launch_selective_scan<bf16_t>((hipStream_t)stream, *c);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Scan with one decay per head.  Per head h (its group g = h / (heads / groups)), token after token:
+//   dt = softplus(dt_raw_h + dt_bias_h);   a = exp(-exp(A_log_h) * dt)
+//   S_h[n][p] <- a * S_h[n][p] + dt * B_g[n] * x_h[p];   y_h[p] = sum_n S_h[n][p] * C_g[n] + D_h * x_h[p]
+// One wave per (4 channels p of a head, sequence): sixteen lanes share a channel, lane j of them owns
+// the state elements j, j + 16, ... in registers.
+struct HeadScanCall {
+  int tokens, n_seqs, heads, vdim, state, groups;
+  const float* x;         // [tokens][ld]: head h at columns h * vdim (after convolution and silu)
+  const float* B;         // [tokens][ld]: group g at columns g * state
+  const float* C;
+  int64_t ld;
+  const float* dt_raw;    // [tokens][ld_dt]: one per head, before bias and softplus
+  int64_t ld_dt;
+  const float* dt_bias;   // [heads]
+  const float* A_log;     // [heads]
+  const float* D;         // [heads]
+  float* y;               // [tokens][ld_y] float32: head h at columns h * vdim
+  int64_t ld_y;
+  float* S;               // slot s: [heads][state][vdim] at S + s * state_stride
+  int64_t state_stride;
+  const int* seq_off;
+  const int* slots;
+};
+
+template <int R, int U>
+__global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c) {
+  const int lane = threadIdx.x, sub = lane & 15;
+  const int p = blockIdx.x * 4 + (lane >> 4), head = blockIdx.y, seq = blockIdx.z;
+  const bool live = p < c.vdim;
+  const int ps = live ? p : c.vdim - 1;
+  const int group = head / (c.heads / c.groups);
+  const int first = c.seq_off[seq], last = c.seq_off[seq + 1];
+  float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + (int64_t)head * c.state * c.vdim + ps;
+  float S[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int n = sub + 16 * r;
+    S[r] = n < c.state ? held[(int64_t)n * c.vdim] : 0.f;
+  }
+  const float rate = -expf(c.A_log[head]), bias = c.dt_bias[head], Dh = c.D[head];
+  const float* xcol = c.x + head * c.vdim + ps;
+  const float* Bg = c.B + group * c.state;
+  const float* Cg = c.C + group * c.state;
+  for (int t0 = first; t0 < last; t0 += U) {
+    float dt[U], xv[U], Bv[U][R], Cv[U][R];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int t = min(t0 + u, last - 1);
+      dt[u] = c.dt_raw[(int64_t)t * c.ld_dt + head];
+      xv[u] = xcol[(int64_t)t * c.ld];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int n = sub + 16 * r;
+        Bv[u][r] = n < c.state ? Bg[(int64_t)t * c.ld + n] : 0.f;
+        Cv[u][r] = n < c.state ? Cg[(int64_t)t * c.ld + n] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (t0 + u < last) {
+        const float step = softplus_f(dt[u] + bias);
+        const float decay = expf(rate * step), dx = step * xv[u];
+        float acc = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          S[r] = decay * S[r] + dx * Bv[u][r];
+          acc = fmaf(S[r], Cv[u][r], acc);
+        }
+        acc += __shfl_xor(acc, 8, 64);
+        acc += __shfl_xor(acc, 4, 64);
+        acc += __shfl_xor(acc, 2, 64);
+        acc += __shfl_xor(acc, 1, 64);
+        if (live && sub == 0) c.y[(int64_t)(t0 + u) * c.ld_y + head * c.vdim + p] = acc + Dh * xv[u];
+      }
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = sub + 16 * r;
+      if (n < c.state) held[(int64_t)n * c.vdim] = S[r];
+    }
+  }
+}
+
+BT_EXPORT int bt_head_scan_call(void* stream, const HeadScanCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->heads <= 0 || c->vdim <= 0 || c->state <= 0 || c->state > 256 || c->groups <= 0 || c->heads % c->groups != 0 || c->n_seqs <= 0)
+    BT_REFUSE("head_scan: %d heads of %d in %d groups with %d state elements (1..256)", c->heads, c->vdim, c->groups, c->state);
+  if (!c->x || !c->B || !c->C || !c->dt_raw || !c->dt_bias || !c->A_log || !c->D || !c->y || !c->S || !c->seq_off || !c->slots)
+    BT_REFUSE("head_scan: missing operand");
+  if (c->ld_dt < c->heads || c->ld_y < (int64_t)c->heads * c->vdim ||
+      c->state_stride < (int64_t)c->heads * c->state * c->vdim)
+    BT_REFUSE("head_scan: rows or state too short for %d heads of %d", c->heads, c->vdim);
+  dim3 grid((c->vdim + 3) / 4, c->heads, c->n_seqs), block(64);
+  hipStream_t s = (hipStream_t)stream;
+  const int per = (c->state + 15) / 16;
+  if (per <= 1) hipLaunchKernelGGL((head_scan_kernel<1, 8>), grid, block, 0, s, *c);
+  else if (per <= 2) hipLaunchKernelGGL((head_scan_kernel<2, 8>), grid, block, 0, s, *c);
+  else if (per <= 4) hipLaunchKernelGGL((head_scan_kernel<4, 4>), grid, block, 0, s, *c);
+  else if (per <= 8) hipLaunchKernelGGL((head_scan_kernel<8, 2>), grid, block, 0, s, *c);
+  else hipLaunchKernelGGL((head_scan_kernel<16, 1>), grid, block, 0, s, *c);
+  return bt_check_launch("head_scan");
+}
+
+// ---------------------------------------------------------------------------------------------
+// v = y * silu(z); out = v / sqrt(mean(v^2) + eps) * weight, the mean over each of `parts` equal
+// parts of the row on its own.
+struct GatedNormCall {
+  int out_dtype;
+  int tokens, channels, parts;
+  int out_cols;           // columns of out written: the channels, then zeros
+  float eps;
+  const float* y;         // [tokens][ld_y]
+  int64_t ld_y;
+  const float* z;         // [tokens][ld_z] gate, pre-activation
+  int64_t ld_z;
+  const float* weight;    // [channels]
+  void* out;              // [tokens][ld_out]
+  int64_t ld_out;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) gated_norm_kernel(GatedNormCall c) {
+  extern __shared__ float row_buf[];
+  __shared__ float scratch[32];
+  const int t = blockIdx.x, part = blockIdx.y;
+  const int n = c.channels / c.parts, base = part * n;
+  float partial = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float v = c.y[(int64_t)t * c.ld_y + base + i] * silu_f(c.z[(int64_t)t * c.ld_z + base + i]);
+    row_buf[i] = v;
+    partial += v * v;
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(partial, scratch) / (float)n + c.eps);
+  T* out = static_cast<T*>(c.out) + (int64_t)t * c.ld_out;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) out[base + i] = from_float<T>(row_buf[i] * rstd * c.weight[base + i]);
+  if (part == 0)
+    for (int col = c.channels + threadIdx.x; col < c.out_cols; col += blockDim.x) out[col] = from_float<T>(0.f);
+}
+
+BT_EXPORT int bt_gated_norm_call(void* stream, const GatedNormCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->channels <= 0 || c->parts <= 0 || c->channels % c->parts != 0 || c->channels / c->parts > 15360)
+    BT_REFUSE("gated_norm: %d channels in %d equal parts (each up to 15360)", c->channels, c->parts);
+  if (!c->y || !c->z || !c->weight || !c->out || c->ld_y < c->channels || c->ld_z < c->channels ||
+      c->out_cols < c->channels || c->ld_out < c->out_cols)
+    BT_REFUSE("gated_norm: missing operand or rows too short");
+  dim3 grid(c->tokens, c->parts), block(256);
+  size_t lds = (size_t)(c->channels / c->parts) * sizeof(float);
+  if (c->out_dtype == 0)
+    hipLaunchKernelGGL(gated_norm_kernel<float>, grid, block, lds, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(gated_norm_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, *c);
+  return bt_check_launch("gated_norm");
+}

@@ -1,0 +1,134 @@
+// Kernels for layers that normalise a sublayer's OUTPUT before it joins the residual stream, and
+// for activations that are norms themselves.  All statistics and the residual sum are 32-bit.
+//   * output norm: x[t] (+)= mult * v / sqrt(mean(v^2) + eps) * gamma, v the sublayer's output
+//     (the sum of its partial sums and its bias), and a copy of the new x in the products' type
+//   * PolyNorm: a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over a row
+#include "host.h"
+
+struct OutputNormCall {
+  int cast_dtype;        // element type of `cast`: 0 float32, 1 bfloat16
+  int n_delta;           // partial sums of the sublayer's output; 0: the stream's own rows are normalised
+  int tokens;
+  int width;
+  int accumulate;        // 1: x += mult * norm(v); 0: x = mult * norm(v)
+  int cast_cols;         // columns of `cast` that are written: the new x, then zeros
+  float eps;
+  float mult;
+  float* x;              // [tokens][width] float32 residual stream
+  const float* delta;    // [n_delta][..][ldd]
+  int64_t delta_stride;  // elements between two partial sums
+  int64_t ldd;           // row pitch of a partial sum
+  const float* bias;     // [width] or null: added to v
+  const float* gamma;    // [width]
+  void* cast;            // [tokens][ld_cast] or null
+  int64_t ld_cast;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) output_norm_kernel(OutputNormCall c) {
+  extern __shared__ float row_buf[];
+  __shared__ float scratch[32];
+  const int t = blockIdx.x;
+  float* xr = c.x + (int64_t)t * c.width;
+  float partial = 0.f;
+  for (int col = threadIdx.x; col < c.width; col += blockDim.x) {
+    float v;
+    if (c.n_delta == 0) {
+      v = xr[col];
+    } else {
+      v = c.bias ? c.bias[col] : 0.f;
+      for (int s = 0; s < c.n_delta; ++s) v += c.delta[s * c.delta_stride + (int64_t)t * c.ldd + col];
+    }
+    row_buf[col] = v;
+    partial += v * v;
+  }
+  const float total = block_sum(partial, scratch);
+  const float scale = c.mult / sqrtf(total / (float)c.width + c.eps);
+  T* cast = static_cast<T*>(c.cast);
+  for (int col = threadIdx.x; col < c.width; col += blockDim.x) {
+    float y = row_buf[col] * scale * c.gamma[col];
+    if (c.accumulate) y += xr[col];
+    xr[col] = y;
+    if (cast) cast[(int64_t)t * c.ld_cast + col] = from_float<T>(y);
+  }
+  if (cast)
+    for (int col = c.width + threadIdx.x; col < c.cast_cols; col += blockDim.x)
+      cast[(int64_t)t * c.ld_cast + col] = from_float<T>(0.f);
+}
+
+BT_EXPORT int bt_output_norm_call(void* stream, const OutputNormCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->width <= 0 || c->width > 15360) BT_REFUSE("output_norm: width %d outside 1..15360", c->width);
+  if (!c->x || !c->gamma || (c->n_delta > 0 && !c->delta)) BT_REFUSE("output_norm: missing operand");
+  if (c->n_delta == 0 && c->accumulate) BT_REFUSE("output_norm: the stream's own rows cannot be added to themselves");
+  if (c->cast && (c->cast_cols < c->width || c->ld_cast < c->cast_cols))
+    BT_REFUSE("output_norm: a copy of %d columns in rows of %lld does not hold width %d", c->cast_cols,
+              (long long)c->ld_cast, c->width);
+  dim3 grid(c->tokens), block(256);
+  size_t lds = (size_t)c->width * sizeof(float);
+  if (c->cast_dtype == 0)
+    hipLaunchKernelGGL(output_norm_kernel<float>, grid, block, lds, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(output_norm_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, *c);
+  return bt_check_launch("output_norm");
+}
+
+struct PolyNormCall {
+  int out_dtype;          // 0 float32, 1 bfloat16
+  int tokens;
+  int columns;            // the row's length: statistics are means over these
+  int out_cols;           // columns of `out` that are written: the result, then zeros
+  float eps;
+  const float* z;         // [tokens][ldz] float32
+  int64_t ldz;
+  const float* coefficients;  // a, b, c, e
+  void* out;              // [tokens][ldo]
+  int64_t ldo;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) poly_norm_kernel(PolyNormCall c) {
+  extern __shared__ float row_buf[];
+  __shared__ float scratch[32];
+  const int t = blockIdx.x;
+  const float* zr = c.z + (int64_t)t * c.ldz;
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  for (int col = threadIdx.x; col < c.columns; col += blockDim.x) {
+    const float v = zr[col];
+    row_buf[col] = v;
+    const float v2 = v * v;
+    s2 += v2;
+    s4 += v2 * v2;
+    s6 += v2 * v2 * v2;
+  }
+  s2 = block_sum(s2, scratch);
+  s4 = block_sum(s4, scratch);
+  s6 = block_sum(s6, scratch);
+  const float n = (float)c.columns;
+  const float a = c.coefficients[0] / sqrtf(s2 / n + c.eps);
+  const float b = c.coefficients[1] / sqrtf(s4 / n + c.eps);
+  const float d = c.coefficients[2] / sqrtf(s6 / n + c.eps);
+  const float e = c.coefficients[3];
+  T* out = static_cast<T*>(c.out) + (int64_t)t * c.ldo;
+  for (int col = threadIdx.x; col < c.columns; col += blockDim.x) {
+    const float v = row_buf[col];
+    out[col] = from_float<T>(a * v + b * (v * v) + d * (v * v * v) + e);
+  }
+  for (int col = c.columns + threadIdx.x; col < c.out_cols; col += blockDim.x) out[col] = from_float<T>(0.f);
+}
+
+BT_EXPORT int bt_poly_norm_call(void* stream, const PolyNormCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->columns <= 0 || c->columns > 15360) BT_REFUSE("poly_norm: %d columns outside 1..15360", c->columns);
+  if (!c->z || !c->coefficients || !c->out) BT_REFUSE("poly_norm: missing operand");
+  if (c->out_cols < c->columns || c->ldo < c->out_cols || c->ldz < c->columns)
+    BT_REFUSE("poly_norm: rows of %lld and %lld elements do not hold %d (%d) columns", (long long)c->ldz,
+              (long long)c->ldo, c->columns, c->out_cols);
+  dim3 grid(c->tokens), block(256);
+  size_t lds = (size_t)c->columns * sizeof(float);
+  if (c->out_dtype == 0)
+    hipLaunchKernelGGL(poly_norm_kernel<float>, grid, block, lds, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(poly_norm_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, *c);
+  return bt_check_launch("poly_norm");
+}

@@ -31,12 +31,12 @@ class CausalLM:
         for layer in plan.layers:
             block_class = lookup("block", layer.block)
             unknown = set(layer.parts) - set(block_class.ROLES)
-            absent = set(block_class.ROLES) - set(layer.parts)
+            absent = set(block_class.ROLES) - set(layer.parts) - set(block_class.OPTIONAL)
             if unknown or absent:
                 raise ValueError(f"block {layer.block!r} takes parts {sorted(block_class.ROLES)}, "
                                  f"the plan gives {sorted(layer.parts)}")
-            self.blocks.append(block_class({name: build_part(block_class.ROLES[name], spec, store)
-                                            for name, spec in layer.parts.items()}))
+            parts = {name: build_part(block_class.ROLES[name], spec, store) for name, spec in layer.parts.items()}
+            self.blocks.append(block_class(parts, layer.params) if layer.params else block_class(parts))
         self.final_norm = build_part("norm", plan.final_norm, store)
         self.readout = build_part("readout", plan.readout, store)
         self.schedule = list(plan.schedule)

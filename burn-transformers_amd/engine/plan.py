@@ -20,9 +20,11 @@ class PartSpec:
 
 @dataclass
 class LayerPlan:
-    """One layer: the arrangement of its parts (a block kind) and the parts themselves."""
+    """One layer: the arrangement of its parts (a block kind), the parts themselves, and the
+    arrangement's own constants (``params``; most have none)."""
     block: str
     parts: Dict[str, PartSpec]
+    params: Dict[str, object] = field(default_factory=dict)
 
 
 @dataclass

@@ -83,6 +83,73 @@ class KvCopyCall(ctypes.Structure):
                 ("ld", _c_i64), ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("kv", KvView)]
 
 
+class OutputNormCall(ctypes.Structure):
+    _fields_ = [("cast_dtype", _c_int), ("n_delta", _c_int), ("tokens", _c_int), ("width", _c_int),
+                ("accumulate", _c_int), ("cast_cols", _c_int), ("eps", _c_float), ("mult", _c_float), ("x", _c_ptr),
+                ("delta", _c_ptr), ("delta_stride", _c_i64), ("ldd", _c_i64), ("bias", _c_ptr), ("gamma", _c_ptr),
+                ("cast", _c_ptr), ("ld_cast", _c_i64)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class PolyNormCall(ctypes.Structure):
+    _fields_ = [("out_dtype", _c_int), ("tokens", _c_int), ("columns", _c_int), ("out_cols", _c_int), ("eps", _c_float),
+                ("z", _c_ptr), ("ldz", _c_i64), ("coefficients", _c_ptr), ("out", _c_ptr), ("ldo", _c_i64)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class LatentNormCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("q_rank", _c_int), ("q_cols", _c_int), ("kv_rank", _c_int),
+                ("kv_offset", _c_int), ("eps", _c_float), ("input", _c_ptr), ("ld", _c_i64), ("q_gamma", _c_ptr),
+                ("kv_gamma", _c_ptr), ("q_out", _c_ptr), ("ld_q", _c_i64), ("tok_seq", _c_ptr), ("tok_pos", _c_ptr),
+                ("kv", KvView)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class HeadProjectCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("heads", _c_int), ("vdim", _c_int), ("rank", _c_int),
+                ("head_pitch", _c_int), ("out_cols", _c_int), ("ctx", _c_ptr), ("ld_ctx", _c_i64), ("W", _c_ptr),
+                ("gate", _c_ptr), ("ld_gate", _c_i64), ("out", _c_ptr), ("ld_out", _c_i64)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class CausalConvCall(ctypes.Structure):
+    _fields_ = [("cast_dtype", _c_int), ("tokens", _c_int), ("n_seqs", _c_int), ("channels", _c_int), ("taps", _c_int),
+                ("cast_cols", _c_int), ("input", _c_ptr), ("ld_in", _c_i64), ("weight", _c_ptr), ("bias", _c_ptr),
+                ("out", _c_ptr), ("ld_out", _c_i64), ("cast", _c_ptr), ("ld_cast", _c_i64), ("state", _c_ptr),
+                ("state_stride", _c_i64), ("tok_seq", _c_ptr), ("seq_off", _c_ptr), ("slots", _c_ptr)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class DtProjectCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("channels", _c_int), ("rank", _c_int), ("low", _c_ptr),
+                ("ld_low", _c_i64), ("W", _c_ptr), ("bias", _c_ptr), ("out", _c_ptr), ("ld_out", _c_i64)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class SelectiveScanCall(ctypes.Structure):
+    _fields_ = [("out_dtype", _c_int), ("tokens", _c_int), ("n_seqs", _c_int), ("channels", _c_int), ("state", _c_int),
+                ("out_cols", _c_int), ("x", _c_ptr), ("ld_x", _c_i64), ("z", _c_ptr), ("ld_z", _c_i64), ("dt", _c_ptr),
+                ("ld_dt", _c_i64), ("B", _c_ptr), ("C", _c_ptr), ("ld_bc", _c_i64), ("A_log", _c_ptr), ("D", _c_ptr),
+                ("out", _c_ptr), ("ld_out", _c_i64), ("S", _c_ptr), ("state_stride", _c_i64), ("seq_off", _c_ptr),
+                ("slots", _c_ptr)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class HeadScanCall(ctypes.Structure):
+    _fields_ = [("tokens", _c_int), ("n_seqs", _c_int), ("heads", _c_int), ("vdim", _c_int), ("state", _c_int),
+                ("groups", _c_int), ("x", _c_ptr), ("B", _c_ptr), ("C", _c_ptr), ("ld", _c_i64), ("dt_raw", _c_ptr),
+                ("ld_dt", _c_i64), ("dt_bias", _c_ptr), ("A_log", _c_ptr), ("D", _c_ptr), ("y", _c_ptr),
+                ("ld_y", _c_i64), ("S", _c_ptr), ("state_stride", _c_i64), ("seq_off", _c_ptr), ("slots", _c_ptr)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class GatedNormCall(ctypes.Structure):
+    _fields_ = [("out_dtype", _c_int), ("tokens", _c_int), ("channels", _c_int), ("parts", _c_int), ("out_cols", _c_int),
+                ("eps", _c_float), ("y", _c_ptr), ("ld_y", _c_i64), ("z", _c_ptr), ("ld_z", _c_i64), ("weight", _c_ptr),
+                ("out", _c_ptr), ("ld_out", _c_i64)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
 class LaunchEntry(ctypes.Structure):
     _fields_ = [("call", _c_ptr), ("args", _c_ptr)]
 
@@ -899,3 +966,123 @@ def count_tokens(counts, rows, tokens):
     pairs = torch.tensor([list(rows), list(tokens)], dtype=torch.int32).to(counts.device, non_blocking=True)
     _check(lib, lib.bt_count_tokens(_c_ptr(_stream()), _c_ptr(counts.data_ptr()), _c_i64(counts.stride(0)),
                                     _c_ptr(pairs[0].data_ptr()), _c_ptr(pairs[1].data_ptr()), _c_int(len(rows))))
+
+
+# --- norms of a sublayer's output, activations that are norms ---------------------------------
+
+def output_norm(x, gamma, eps, mult=1.0, delta=None, bias=None, accumulate=True, cast=None):
+    """x[t] (+)= mult * v / sqrt(mean(v^2) + eps) * gamma with v = sum(delta[:, t]) + bias (``delta``
+    float32 [splits, tokens, width] or [tokens, width]); without ``delta`` the stream's own rows are
+    normalised in place (``accumulate`` must then be False).  ``cast``: a tensor [tokens, >= width]
+    in the products' type that receives the new x (and zeros behind it)."""
+    tokens, width = x.shape
+    if delta is None:
+        n_delta, stride, ldd = 0, 0, 0
+    elif delta.dim() == 3:
+        n_delta, stride, ldd = delta.shape[0], delta.stride(0), delta.stride(1)
+    else:
+        n_delta, stride, ldd = 1, 0, delta.stride(0)
+    _launch(_module("sublayer"), "bt_output_norm_call",
+            OutputNormCall(cast_dtype=DTYPE_CODES[cast.dtype] if cast is not None else FLOAT32, n_delta=n_delta,
+                           tokens=tokens, width=width, accumulate=1 if accumulate else 0,
+                           cast_cols=cast.shape[1] if cast is not None else 0, eps=eps, mult=mult, x=x.data_ptr(),
+                           delta=_ptr(delta), delta_stride=stride, ldd=ldd, bias=_ptr(bias), gamma=gamma.data_ptr(),
+                           cast=_ptr(cast), ld_cast=cast.stride(0) if cast is not None else 0))
+
+
+def poly_norm(z, columns, coefficients, eps, out):
+    """out = a N(z) + b N(z^2) + c N(z^3) + e over the first ``columns`` of each float32 row of ``z``,
+    N(v) = v / sqrt(mean(v^2) + eps); (a, b, c, e) = ``coefficients`` (float32 on the GPU).  The
+    columns of ``out`` behind them are set to zero."""
+    _launch(_module("sublayer"), "bt_poly_norm_call",
+            PolyNormCall(out_dtype=DTYPE_CODES[out.dtype], tokens=z.shape[0], columns=columns, out_cols=out.shape[1],
+                         eps=eps, z=z.data_ptr(), ldz=z.stride(0), coefficients=coefficients.data_ptr(),
+                         out=out.data_ptr(), ldo=out.stride(0)))
+
+
+# --- latent attention ------------------------------------------------------------------------
+
+def latent_norm(fused, q_rank, kv_offset, kv_rank, q_gamma, kv_gamma, eps, q_out, tok_seq, tok_pos, kv_view, dtype):
+    """The two RMS norms behind a fused down-projection (float32 rows ``fused``): columns [0, q_rank)
+    go normalised to ``q_out`` (zeros behind them), columns [kv_offset, kv_offset + kv_rank) into the
+    paged cache at each token's position, as the keys AND the values of its one head."""
+    _launch(_module("latent"), "bt_latent_norm_call",
+            LatentNormCall(dtype=DTYPE_CODES[dtype], tokens=fused.shape[0], q_rank=q_rank, q_cols=q_out.shape[1],
+                           kv_rank=kv_rank, kv_offset=kv_offset, eps=eps, input=fused.data_ptr(), ld=fused.stride(0),
+                           q_gamma=q_gamma.data_ptr(), kv_gamma=kv_gamma.data_ptr(), q_out=q_out.data_ptr(),
+                           ld_q=q_out.stride(0), tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), kv=kv_view))
+
+
+def head_project(ctx, weight, heads, vdim, rank, head_pitch, out, gate=None):
+    """out[t, h * vdim + v] = sigmoid(gate[t, h * vdim + v]) * sum_r weight[h * vdim + v, r] * ctx[t, h * head_pitch + r]
+    (without ``gate``: no factor); the columns of ``out`` behind heads * vdim are set to zero."""
+    if ctx.dtype != weight.dtype or out.dtype != weight.dtype or not weight.is_contiguous() or \
+            tuple(weight.shape) != (heads * vdim, rank):
+        raise KernelError(f"head_project: weights {tuple(weight.shape)} {weight.dtype} do not fit {heads} heads of {vdim} from rank {rank}")
+    _launch(_module("latent"), "bt_head_project_call",
+            HeadProjectCall(dtype=DTYPE_CODES[weight.dtype], tokens=ctx.shape[0], heads=heads, vdim=vdim, rank=rank,
+                            head_pitch=head_pitch, out_cols=out.shape[1], ctx=ctx.data_ptr(), ld_ctx=ctx.stride(0),
+                            W=weight.data_ptr(), gate=_ptr(gate), ld_gate=gate.stride(0) if gate is not None else 0,
+                            out=out.data_ptr(), ld_out=out.stride(0)))
+
+
+# --- recurrent mixers ------------------------------------------------------------------------
+
+def causal_conv(rows, weight, bias, out, state, step, cast=None):
+    """out = silu(bias + sum_j weight[:, j] * rows[t - (taps - 1 - j)]) per channel and sequence
+    (float32); inputs before a step's first token come from ``state`` ([slots, >= (taps - 1) *
+    channels] float32, oldest first), which then takes the step's last taps - 1 inputs.  ``cast``:
+    the same result in the products' type (zeros behind the channels)."""
+    channels, taps = weight.shape
+    _launch(_module("state_space"), "bt_causal_conv_call",
+            CausalConvCall(cast_dtype=DTYPE_CODES[cast.dtype] if cast is not None else FLOAT32, tokens=rows.shape[0],
+                           n_seqs=step.n_seqs, channels=channels, taps=taps,
+                           cast_cols=cast.shape[1] if cast is not None else 0, input=rows.data_ptr(),
+                           ld_in=rows.stride(0), weight=weight.data_ptr(), bias=bias.data_ptr(), out=out.data_ptr(),
+                           ld_out=out.stride(0), cast=_ptr(cast), ld_cast=cast.stride(0) if cast is not None else 0,
+                           state=state.data_ptr(), state_stride=state.stride(0), tok_seq=step.tok_seq.data_ptr(),
+                           seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr()))
+
+
+def dt_project(low, weight, bias, out):
+    """out = softplus(low . weight^T + bias) in float32; ``low`` float32 [tokens, rank] (rows may be
+    strided), ``weight`` [channels, rank]."""
+    _launch(_module("state_space"), "bt_dt_project_call",
+            DtProjectCall(dtype=DTYPE_CODES[weight.dtype], tokens=low.shape[0], channels=weight.shape[0],
+                          rank=weight.shape[1], low=low.data_ptr(), ld_low=low.stride(0), W=weight.data_ptr(),
+                          bias=bias.data_ptr(), out=out.data_ptr(), ld_out=out.stride(0)))
+
+
+def selective_scan(x, z, dt, B, C, A_log, D, out, state, step):
+    """The selective scan with one state row per channel (see csrc/state_space.hip), gated by
+    silu(z); ``state`` [slots, >= channels * state elements] float32 is read and left updated."""
+    channels, elements = A_log.shape
+    _launch(_module("state_space"), "bt_selective_scan_call",
+            SelectiveScanCall(out_dtype=DTYPE_CODES[out.dtype], tokens=x.shape[0], n_seqs=step.n_seqs, channels=channels,
+                              state=elements, out_cols=out.shape[1], x=x.data_ptr(), ld_x=x.stride(0), z=z.data_ptr(),
+                              ld_z=z.stride(0), dt=dt.data_ptr(), ld_dt=dt.stride(0), B=B.data_ptr(), C=C.data_ptr(),
+                              ld_bc=B.stride(0), A_log=A_log.data_ptr(), D=D.data_ptr(), out=out.data_ptr(),
+                              ld_out=out.stride(0), S=state.data_ptr(), state_stride=state.stride(0),
+                              seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr()))
+
+
+def head_scan(x, B, C, dt_raw, dt_bias, A_log, D, y, state, step, heads, vdim, elements, groups):
+    """The scan with one decay per head (see csrc/state_space.hip); x, B and C are column ranges of
+    the same float32 rows; ``state`` [slots, >= heads * elements * vdim] float32."""
+    if x.stride(0) != B.stride(0) or x.stride(0) != C.stride(0):
+        raise KernelError("head_scan: x, B and C must be column ranges of the same rows")
+    _launch(_module("state_space"), "bt_head_scan_call",
+            HeadScanCall(tokens=x.shape[0], n_seqs=step.n_seqs, heads=heads, vdim=vdim, state=elements, groups=groups,
+                         x=x.data_ptr(), B=B.data_ptr(), C=C.data_ptr(), ld=x.stride(0), dt_raw=dt_raw.data_ptr(),
+                         ld_dt=dt_raw.stride(0), dt_bias=dt_bias.data_ptr(), A_log=A_log.data_ptr(), D=D.data_ptr(),
+                         y=y.data_ptr(), ld_y=y.stride(0), S=state.data_ptr(), state_stride=state.stride(0),
+                         seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr()))
+
+
+def gated_norm(y, z, weight, parts, eps, out):
+    """out = v / sqrt(mean(v^2) + eps) * weight with v = y * silu(z), each of ``parts`` equal parts of
+    a row by its own mean; zeros behind the channels."""
+    _launch(_module("state_space"), "bt_gated_norm_call",
+            GatedNormCall(out_dtype=DTYPE_CODES[out.dtype], tokens=y.shape[0], channels=weight.shape[0], parts=parts,
+                          out_cols=out.shape[1], eps=eps, y=y.data_ptr(), ld_y=y.stride(0), z=z.data_ptr(),
+                          ld_z=z.stride(0), weight=weight.data_ptr(), out=out.data_ptr(), ld_out=out.stride(0)))

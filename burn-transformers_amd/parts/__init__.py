@@ -1,4 +1,5 @@
-from . import attention, block, feed_forward, norm, position, readout  # noqa: F401  (registers the parts)
+from . import (attention, block, feed_forward, latent_attention, norm, position, readout,  # noqa: F401  (registers the parts)
+               state_space)
 from .base import (Block, Delta, Embedding, FeedForward, Memory, Mixer, Norm, Part, Readout,
                    ResidualStream)
 from .registry import lookup, register, unregister

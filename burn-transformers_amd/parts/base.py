@@ -42,11 +42,28 @@ class ResidualStream:
         # set by a block around a part whose output the next norm wants in the stream itself, not
         # pending beside it (the norm is then folded into the product that follows it)
         self.in_place = False
+        # the same rows in the products' type (bfloat16 models), kept up to date by whoever changes x
+        # together with x; None where nobody keeps one.  Parts that read the stream itself, not a
+        # norm of it, multiply by this (``operand``).
+        self.cast = None
+
+    def operand(self, step):
+        """The stream's rows as a product's operand: x itself in float32 models, its copy in the
+        products' type otherwise."""
+        if self.cast is not None:
+            return self.cast
+        if self.pending is not None:
+            self.flush()
+        if step.dtype != self.x.dtype:
+            raise ValueError("the residual stream has no copy in the products' type here: the part that "
+                             "changed it last (an embedding, a norm of outputs) keeps one, others do not")
+        return self.x
 
     def add(self, delta):
         if self.pending is not None:
             self.flush()
         self.pending = delta
+        self.cast = None            # x is about to change, its copy is not
 
     def add_product(self, step, a, weight, bias=None, packed=None):
         """x += a . weight^T + bias.  In a decode step (up to 64 rows) a product with few
@@ -55,24 +72,14 @@ class ResidualStream:
         chunk (``kernels.library.deep_split_count``).  Otherwise the product's epilogue adds into the
         stream in place.  ``packed``: the weight's ``kernels.library.PackedWeight``, if it has one."""
         rows, width = a.shape[0], weight.shape[0]
-        if self.in_place:
-            splits = 1
-        elif step.dtype_is_bf16 and rows > 64:       # a short prompt or chunk: the tile kernel's deep forms
-            splits = K.deep_split_count(rows, width, a.shape[1], compute_units(a.device)) \
-                if not isinstance(a, K.Chunked) and a.stride(1) == 1 and \
-                K.deep_form_rows(rows, a.shape[1], a.stride(0), width, sliced=True) else 1
-        elif step.dtype_is_bf16:
-            splits = split_count(rows, width, a.shape[1], compute_units(a.device), 32)
-        elif a.shape[1] % 4 == 0 and a.stride(0) % 4 == 0:        # what the float32 MFMA kernels take
-            splits = split_count(rows, width, a.shape[1], compute_units(a.device), 16)
-        else:
-            splits = 1
+        splits = 1 if self.in_place else stream_product_splits(step, a, weight)
         if splits > 1:
             partials = step.partial_sums("stream.partials", splits, rows, width)
             K.gemm(a, weight, K.epilogue_f32(partials), splits=splits, packed=packed)
             self.add(Delta(partials, bias))
         else:
             self.flush()
+            self.cast = None
             K.gemm(a, weight, K.epilogue_residual(self.x, bias), packed=packed)
 
     def flush(self):
@@ -80,6 +87,49 @@ class ResidualStream:
         if self.pending is not None:
             K.add_norm(self.x, None, None, None, 0.0, delta=self.pending.partials, bias=self.pending.bias)
             self.pending = None
+
+
+def stream_product_splits(step, a, weight):
+    """Into how many slices of K a product that feeds the residual stream is cut (see
+    ``ResidualStream.add_product``)."""
+    rows, width = a.shape[0], weight.shape[0]
+    if step.dtype_is_bf16 and rows > 64:       # a short prompt or chunk: the tile kernel's deep forms
+        return K.deep_split_count(rows, width, a.shape[1], compute_units(a.device)) \
+            if not isinstance(a, K.Chunked) and a.stride(1) == 1 and \
+            K.deep_form_rows(rows, a.shape[1], a.stride(0), width, sliced=True) else 1
+    if step.dtype_is_bf16:
+        return split_count(rows, width, a.shape[1], compute_units(a.device), 32)
+    if a.shape[1] % 4 == 0 and a.stride(0) % 4 == 0:        # what the float32 MFMA kernels take
+        return split_count(rows, width, a.shape[1], compute_units(a.device), 16)
+    return 1
+
+
+class SublayerOutput(ResidualStream):
+    """Stands where the residual stream would for a part whose OUTPUT is normalised before it joins
+    the stream (``parts.block.OutputNormBlock``): what the part adds is kept as 32-bit partial sums
+    (a ``Delta``), never added to anything, and the block hands it to the norm.  Parts written for the
+    residual stream (``stream.add_product``, ``stream.add``, or a returned ``Delta``) run unchanged."""
+
+    def __init__(self):
+        super().__init__(None)
+
+    def add(self, delta):
+        if self.pending is not None:
+            raise ValueError("a sublayer leaves one output; a second contribution came")
+        self.pending = delta
+
+    def add_product(self, step, a, weight, bias=None, packed=None):
+        splits = stream_product_splits(step, a, weight)
+        partials = step.partial_sums("sublayer.partials", splits, a.shape[0], weight.shape[0])
+        K.gemm(a, weight, K.epilogue_f32(partials), splits=splits, packed=packed)
+        self.add(Delta(partials, bias))
+
+    def flush(self):
+        raise ValueError("a sublayer's output is handed to the norm behind it, not added to the stream")
+
+    def take(self):
+        delta, self.pending = self.pending, None
+        return delta
 
 
 class Memory:
@@ -191,10 +241,11 @@ class Block:
     the engine asks the block, not the names, what it needs."""
 
     ROLES = {}
+    OPTIONAL = ()                       # roles a layer may leave out
     only_launches_kernels = False       # as for a part: True if ``forward`` only calls its parts and the stream
 
-    def __init__(self, parts):
-        self.parts = parts
+    def __init__(self, parts, params=None):
+        self.parts, self.params = parts, dict(params or {})
 
     def recordable(self):
         """Whether a step of this block can be kept as a launch list."""
@@ -223,6 +274,28 @@ class Block:
 @functools.lru_cache(maxsize=None)
 def compute_units(device):
     return torch.cuda.get_device_properties(device).multi_processor_count
+
+
+def operand_columns(count, dtype):
+    """Columns of a buffer that holds ``count`` values per row and is read as a product's operand:
+    the bfloat16 MFMA kernels read 16 bytes at a time, so rows and K are multiples of eight there
+    (the columns behind ``count`` hold zeros and meet zero columns of the weights); float32 operands
+    of any length run (on the plain kernel where they are no multiple of four)."""
+    return (count + 7) // 8 * 8 if dtype == torch.bfloat16 else count
+
+
+def pad_rows(weight, rows):
+    """``weight`` [n, k] with zero rows appended up to ``rows``."""
+    if weight.shape[0] == rows:
+        return weight.contiguous()
+    return torch.cat([weight, weight.new_zeros(rows - weight.shape[0], weight.shape[1])]).contiguous()
+
+
+def pad_columns(weight, columns):
+    """``weight`` [n, k] with zero columns appended up to ``columns``."""
+    if weight.shape[1] == columns:
+        return weight.contiguous()
+    return torch.cat([weight, weight.new_zeros(weight.shape[0], columns - weight.shape[1])], dim=1).contiguous()
 
 
 def packed_for_stream(weight):

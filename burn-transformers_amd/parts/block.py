@@ -3,9 +3,13 @@
 pre_norm: y = x + mixer(norm(x)); z = y + feed_forward(norm(y))
 (src/models/gpt2/model.rs:218-270).  A part adds its contribution to the stream itself or
 returns it as a Delta, which stays pending until the next norm reads the stream.
+
+output_norm: y = x + m * norm(mixer(x)); z = y + m * norm(feed_forward(y)), the feed-forward
+optional.  The parts read the stream itself; what is normalised is what they add.  ``m`` is the
+block's parameter ``mult``.
 """
 
-from .base import Block, offers_chunked
+from .base import Block, SublayerOutput, offers_chunked
 from .registry import register
 
 # Most rows of a step whose first norm is folded too.  Measured at GPT-2 XL sizes, ms a decode step
@@ -61,3 +65,31 @@ def _apply(norm, stream, step, only_multiplied):
 def _can_defer(norm, step, rows):
     possible = getattr(norm, "deferred_possible", None)
     return possible is not None and possible(step, rows)
+
+
+@register("block", "output_norm")
+class OutputNormBlock(Block):
+    """Sublayers that read the residual stream as it is and whose outputs are normalised (and scaled
+    by ``mult``) before they join it.  The norms are of a kind with ``add_output`` (rms_norm).  A
+    layer without a feed-forward leaves ``ff`` and ``ff_norm`` out."""
+    ROLES = {"mixer": "mixer", "mixer_norm": "norm", "ff": "feed_forward", "ff_norm": "norm"}
+    OPTIONAL = ("ff", "ff_norm")
+    only_launches_kernels = True
+
+    def __init__(self, parts, params=None):
+        super().__init__(parts, params)
+        self.mult = float(self.params.get("mult", 1.0))
+        if ("ff" in parts) != ("ff_norm" in parts):
+            raise ValueError("output_norm block: a feed-forward and its norm come together")
+        for name in ("mixer_norm", "ff_norm"):
+            if name in parts and not hasattr(parts[name], "add_output"):
+                raise ValueError(f"output_norm block: {type(parts[name]).__name__} cannot normalise a sublayer's output")
+
+    def forward(self, stream, step, memory):
+        parts = self.parts
+        output = SublayerOutput()
+        delta = parts["mixer"].forward(stream.operand(step), step, memory, output)
+        parts["mixer_norm"].add_output(stream, step, delta if delta is not None else output.take(), self.mult)
+        if "ff" in parts:
+            delta = parts["ff"].forward(stream.operand(step), step, output)
+            parts["ff_norm"].add_output(stream, step, delta if delta is not None else output.take(), self.mult)

@@ -5,6 +5,11 @@ Parameters: width, inner, activation ("gelu_tanh": 0.5x(1+tanh(sqrt(2/pi)(x+0.04
 inside the up projection's epilogue (src/feed_forward.rs:397-406 widens half inputs too); the
 down projection adds into the residual stream.
 
+"poly_norm" is an activation that is a norm: a N(z) + b N(z^2) + c N(z^3) + e with powers taken
+element by element and N(v) = v / sqrt(mean(v^2) + eps) over a token's whole inner vector; the four
+numbers are the tensor ``act_coefficients``, ``eps`` a parameter.  It needs a whole row, so the up
+projection leaves 32-bit sums and a kernel of its own applies it.
+
 The MFMA kernels read operands 16 bytes at a time, so an inner width that is no multiple of 8 is
 padded once, when the part is built: zero rows (and zero bias) in the up projection give
 act(0) = 0 in the padded columns, which meet zero columns of the down projection.
@@ -25,8 +30,12 @@ class DenseFeedForward(FeedForward):
     def __init__(self, params, tensors):
         super().__init__(params, tensors)
         self.width, self.inner, self.activation = params["width"], params["inner"], params["activation"]
-        if self.activation not in K.ACTIVATIONS:
+        if self.activation not in K.ACTIVATIONS and self.activation != "poly_norm":
             raise ValueError(f"feed-forward: unknown activation {self.activation!r}")
+        if self.activation == "poly_norm":
+            self.coefficients, self.eps = tensors["act_coefficients"], float(params["eps"])
+            if tuple(self.coefficients.shape) != (4,):
+                raise ValueError(f"feed-forward: poly_norm takes four numbers, got {tuple(self.coefficients.shape)}")
         self.up_weight, self.up_bias = tensors["up_weight"], tensors.get("up_bias")
         self.down_weight, self.down_bias = tensors["down_weight"], tensors.get("down_bias")
         if tuple(self.up_weight.shape) != (self.inner, self.width) or \
@@ -49,6 +58,13 @@ class DenseFeedForward(FeedForward):
 
     def forward(self, h, step, stream):
         tokens = h.shape[0]
+        if self.activation == "poly_norm":
+            z = step.buffer("feed_forward.sums", tokens, self.padded, "float32")
+            hidden = step.buffer("feed_forward.hidden", tokens, self.padded, step.dtype)
+            K.gemm(h, self.up_weight, K.epilogue_f32(z, self.up_bias), packed=self.up_packed)
+            K.poly_norm(z, self.inner, self.coefficients, self.eps, hidden)
+            stream.add_product(step, hidden, self.down_weight, self.down_bias, packed=self.down_packed)
+            return
         if K.Chunked.wanted(tokens) and (step.dtype_is_bf16 or self.padded % 4 == 0):
             hidden = K.Chunked.take(step, "feed_forward.hidden", tokens, self.padded, step.dtype)   # read by the next product only
         else:

@@ -1,0 +1,124 @@
+"""Causal attention through low-rank latents, without positions, with an output gate.
+
+Parameters: width, heads, dim (query/key size per head), vdim (value size per head), q_rank,
+kv_rank, scale (multiplies q.k), eps (of the two latent norms).  Tensors, all [out, in]:
+down_q [q_rank, width], q_norm [q_rank], up_q [heads*dim, q_rank], down_kv [kv_rank, width],
+kv_norm [kv_rank], up_k [heads*dim, kv_rank], up_v [heads*vdim, kv_rank], gate [heads*vdim, width],
+out_weight [width, heads*vdim].
+
+With c_q = rms_norm(down_q h) and c = rms_norm(down_kv h), head i has queries q_i = up_q_i c_q,
+keys k_i = up_k_i c and values v_i = up_v_i c.  Both up-projections of c are linear, so
+    q_i . k_i(j) = (up_k_i^T up_q_i c_q) . c(j)        and        sum_j p_j v_i(j) = up_v_i sum_j p_j c(j):
+attention runs on the latent itself.  Only c is cached, as ONE shared head of size kv_rank whose
+keys and values are the same vector, and the heads' queries against it are the grouped-query case
+of the attention kernels (all heads of a token read each cached vector once).  The matrix
+up_k_i^T up_q_i is formed once when the part is built (in float64, rounded to the products' type).
+
+One step: a fused product [down_q; down_kv; gate] h (32-bit sums) -> the two norms, c straight into
+the paged cache -> absorbed queries (one product) -> attention over the cache -> per head up_v and
+sigmoid gate -> output projection (the sublayer's output).
+"""
+
+import torch
+
+from ..cache.storage import KVSpec
+from ..kernels import library as K
+from .attention import CausalSelfAttention
+from .base import Mixer, operand_columns, pad_columns, pad_rows
+from .registry import register
+
+
+@register("mixer", "latent_attention")
+class LatentAttention(Mixer):
+    only_launches_kernels = True
+
+    def __init__(self, params, tensors):
+        super().__init__(params, tensors)
+        p = params
+        self.width, self.heads, self.dim, self.vdim = p["width"], p["heads"], p["dim"], p["vdim"]
+        self.q_rank, self.kv_rank = p["q_rank"], p["kv_rank"]
+        self.scale, self.eps = float(p["scale"]), float(p["eps"])
+        shapes = {"down_q": (self.q_rank, self.width), "q_norm": (self.q_rank,),
+                  "up_q": (self.heads * self.dim, self.q_rank), "down_kv": (self.kv_rank, self.width),
+                  "kv_norm": (self.kv_rank,), "up_k": (self.heads * self.dim, self.kv_rank),
+                  "up_v": (self.heads * self.vdim, self.kv_rank), "gate": (self.heads * self.vdim, self.width),
+                  "out_weight": (self.width, self.heads * self.vdim)}
+        for role, shape in shapes.items():
+            if tuple(tensors[role].shape) != shape:
+                raise ValueError(f"latent attention: {role} is {tuple(tensors[role].shape)}, expected {shape}")
+        dtype = tensors["down_q"].dtype
+        self.bf16 = dtype == torch.bfloat16
+        # the cached head: the latent, padded to what the attention kernels take (zeros that meet zeros)
+        self.head_dim = (self.kv_rank + 15) // 16 * 16
+        if self.head_dim > 256:
+            raise ValueError(f"latent attention: kv_rank {self.kv_rank} is beyond 256, the most any attention kernel here takes")
+        # the MFMA kernels take heads of up to 128 (bfloat16) and up to 16 query heads per cached head
+        # in decode steps; everything else runs on the plain attention kernel
+        self.plain_only = self.bf16 and (self.head_dim > 128 or self.heads > 16)
+        # segments of the fused first product, each padded so that the next starts where 16-byte loads may
+        self.q_cols = operand_columns(self.q_rank, dtype)
+        self.kv_offset = (self.q_rank + 3) // 4 * 4
+        self.gate_offset = self.kv_offset + (self.kv_rank + 3) // 4 * 4
+        self.fused_cols = self.gate_offset + self.heads * self.vdim
+        self.fused_weight = torch.cat([pad_rows(tensors["down_q"], self.kv_offset),
+                                       pad_rows(tensors["down_kv"], self.gate_offset - self.kv_offset),
+                                       tensors["gate"]]).contiguous()
+        self.q_norm, self.kv_norm = tensors["q_norm"], tensors["kv_norm"]
+        # absorbed queries: rows i * head_dim .. of W are up_k_i^T up_q_i  ([kv_rank, q_rank])
+        up_q = tensors["up_q"].double().view(self.heads, self.dim, self.q_rank)
+        up_k = tensors["up_k"].double().view(self.heads, self.dim, self.kv_rank)
+        absorbed = torch.einsum("hdr,hdq->hrq", up_k, up_q)
+        full = absorbed.new_zeros(self.heads, self.head_dim, self.q_cols)
+        full[:, :self.kv_rank, :self.q_rank] = absorbed
+        self.query_weight = full.view(self.heads * self.head_dim, self.q_cols).to(dtype).contiguous()
+        self.up_v = tensors["up_v"].contiguous()
+        self.mixed_cols = operand_columns(self.heads * self.vdim, dtype)
+        self.out_weight = pad_columns(tensors["out_weight"], self.mixed_cols)
+        self.n_q = self.heads * self.head_dim
+
+    def kv_spec(self):
+        return KVSpec(1, self.head_dim, 0)
+
+    def kernel_modules(self, dtype):
+        names = ["latent"]
+        if not self.plain_only:
+            if dtype == torch.bfloat16:
+                names.append(f"attention_bf16_hd{self.head_dim}")
+            elif self.head_dim <= 128:
+                names.append("attention_f32")
+        return tuple(names)
+
+    # the planning of runs of keys is the ordinary attention's: one cached head, ``heads`` query heads
+    kv_heads = 1
+    window = 0
+    decode_runs = CausalSelfAttention.decode_runs
+    prompt_runs = CausalSelfAttention.prompt_runs
+
+    def forward(self, h, step, memory, stream):
+        tokens = h.shape[0]
+        kv = memory.kv()
+        fused = step.buffer("latent.fused", tokens, self.fused_cols, "float32")
+        K.gemm(h, self.fused_weight, K.epilogue_f32(fused))
+        c_q = step.buffer("latent.query_latent", tokens, self.q_cols, step.dtype)
+        if not memory.writes:
+            raise ValueError("latent attention: every run keeps a cache entry of its own")
+        K.latent_norm(fused, self.q_rank, self.kv_offset, self.kv_rank, self.q_norm, self.kv_norm, self.eps, c_q,
+                      step.tok_seq, step.tok_pos, kv, step.dtype)
+        q = step.buffer("latent.queries", tokens, self.n_q, step.dtype)
+        K.gemm(c_q, self.query_weight, K.epilogue_store(q))
+        ctx = step.buffer("latent.context", tokens, self.n_q, step.dtype)
+        partial, runs, prompt_runs = None, self.decode_runs(step, h.device), self.prompt_runs(step, h.device)
+        if self.plain_only:
+            runs = prompt_runs = 1
+        if runs > 1:
+            partial = step.buffer("attention.partial", step.n_seqs * self.heads * runs, self.head_dim + 2, "float32")
+        elif prompt_runs > 1:
+            partial = step.buffer("attention.partial", tokens * self.heads * prompt_runs, self.head_dim + 2, "float32")
+        args = K.attention_args(q, ctx, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start, self.heads,
+                                step.n_seqs, step.max_count, self.scale, 0, partial,
+                                runs=prompt_runs if prompt_runs > 1 else None)
+        K.attention(args, step.dtype, step.decode, impl="plain" if self.plain_only else "auto")
+        mixed = step.buffer("latent.mixed", tokens, self.mixed_cols, step.dtype)
+        K.head_project(ctx, self.up_v, self.heads, self.vdim, self.kv_rank, self.head_dim, mixed,
+                       gate=fused[:, self.gate_offset:])
+        stream.add_product(step, mixed, self.out_weight)

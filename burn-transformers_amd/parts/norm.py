@@ -4,11 +4,17 @@ layer_norm: y = (x - mean) / sqrt(var + eps) * weight + bias, var the population
             (src/models/gpt2/model.rs:8, 143-148).
 rms_norm:   y = x / sqrt(mean(x^2) + eps) * weight   (src/normalization.rs:158-171).
 
-``apply`` first adds what is pending on the residual stream, in the same pass.
+Parameter ``offset`` (default 0): the scale is stored as its distance from ``offset`` and the norm
+multiplies by offset + weight (1 for scales stored around zero); the sum is formed once, in
+float32, when the part is built.
+
+``apply`` first adds what is pending on the residual stream, in the same pass.  ``add_output``
+(rms_norm) is the norm of a sublayer's OUTPUT: x += mult * norm(output), for layers that read the
+stream itself and normalise what they add to it.
 """
 
 from ..kernels import library as K
-from .base import Norm
+from .base import Norm, operand_columns
 from .registry import register
 
 
@@ -22,6 +28,9 @@ class _KernelNorm(Norm):
         self.weight, self.bias = tensors["weight"], tensors.get("bias")
         if tuple(self.weight.shape) != (self.width,):
             raise ValueError(f"{self.KIND}: scale is {tuple(self.weight.shape)}, expected {(self.width,)}")
+        self.offset = float(params.get("offset", 0.0))
+        if self.offset:
+            self.weight = (self.weight.float() + self.offset).contiguous()
 
     def apply(self, stream, step, rows=None, chunked=False):
         count = rows.numel() if rows is not None else stream.x.shape[0]
@@ -54,3 +63,16 @@ class LayerNorm(_KernelNorm):
 @register("norm", "rms_norm")
 class RMSNorm(_KernelNorm):
     KIND = "rms_norm"
+
+    def add_output(self, stream, step, delta, mult=1.0, accumulate=True):
+        """x (+)= mult * v / sqrt(mean(v^2) + eps) * scale, v = the sublayer's output ``delta`` (a
+        ``Delta``; None: the stream's own rows, normalised in place).  In a bfloat16 model the new
+        rows are also left as the stream's copy in the products' type (``stream.operand``)."""
+        if stream.pending is not None:
+            stream.flush()
+        cast = None
+        if step.dtype != stream.x.dtype:
+            cast = step.buffer("stream.operand", stream.x.shape[0], operand_columns(self.width, step.dtype), step.dtype)
+        K.output_norm(stream.x, self.weight, self.eps, mult, delta=delta.partials if delta is not None else None,
+                      bias=delta.bias if delta is not None else None, accumulate=accumulate, cast=cast)
+        stream.cast = cast

@@ -2,11 +2,13 @@
 
 learned_positions: x0[t] = tokens[id[t]] + positions[pos[t]]  (src/models/gpt2/model.rs:447-448);
 the table's length bounds a sequence's length.  token_only: x0[t] = tokens[id[t]] (for models
-whose position encoding lives in the mixer).
+whose position encoding lives in the mixer).  normalized_tokens: x0[t] = rms_norm(tokens[id[t]]) with
+a scale of its own (stored as its distance from ``offset``), for models that normalise the
+embedding before the first layer; it also leaves the stream's copy in the products' type.
 """
 
 from ..kernels import library as K
-from .base import Embedding, ResidualStream
+from .base import Embedding, ResidualStream, operand_columns
 from .registry import register
 
 
@@ -43,3 +45,27 @@ class TokenEmbedding(Embedding):
         x = step.buffer("stream.x", step.n_tokens, self.width, "float32")
         K.embed(step.tok_ids, None, self.token_table, None, x)
         return ResidualStream(x)
+
+
+@register("embedding", "normalized_tokens")
+class NormalizedTokenEmbedding(Embedding):
+    only_launches_kernels = True
+
+    def __init__(self, params, tensors):
+        super().__init__(params, tensors)
+        self.width, self.vocab_size = params["width"], params["vocab_size"]
+        self.max_positions = params.get("max_positions", 2 ** 31 - 1)
+        self.eps = float(params["eps"])
+        self.token_table = tensors["tokens"]
+        self.scale = (tensors["norm_weight"].float() + float(params.get("offset", 0.0))).contiguous()
+        if tuple(self.token_table.shape) != (self.vocab_size, self.width) or tuple(self.scale.shape) != (self.width,):
+            raise ValueError("embedding: table or scale do not have the configured sizes")
+
+    def embed(self, step):
+        x = step.buffer("stream.x", step.n_tokens, self.width, "float32")
+        K.embed(step.tok_ids, None, self.token_table, None, x)
+        stream = ResidualStream(x)
+        if step.dtype != x.dtype:
+            stream.cast = step.buffer("stream.operand", step.n_tokens, operand_columns(self.width, step.dtype), step.dtype)
+        K.output_norm(x, self.scale, self.eps, 1.0, accumulate=False, cast=stream.cast)
+        return stream
