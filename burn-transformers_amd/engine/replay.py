@@ -61,6 +61,14 @@ class Replay:
             print(f"done {record['step']}", file=out, flush=True)
 
 
+def cache_tokens(max_tokens, block=64, most_requests=256):
+    """Room to give the cache for a trace whose live requests hold ``max_tokens`` tokens: the cache
+    hands out whole blocks, so every live request may hold up to a block less one of room it does not
+    use; there are at most ``max_tokens`` live requests, and more than ``most_requests`` at a time are
+    not provided for."""
+    return max_tokens + (block - 1) * min(max(max_tokens, 1), most_requests)
+
+
 def main(argv=None):
     import argparse
     parser = argparse.ArgumentParser(prog="trace_run", description="Replay a trace of token ids and write logits.")
@@ -68,13 +76,13 @@ def main(argv=None):
     parser.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     parser.add_argument("--out", required=True, help="folder for <step>.f32 files")
     parser.add_argument("--max-tokens", type=int, required=True,
-                        help="most tokens live requests hold at any time (each rounded up to 64)")
+                        help="most tokens live requests hold at any time")
     args = parser.parse_args(argv)
     from .. import Engine, load_model
     print(f"[trace_run] loading {args.model} ({args.dtype}); kernels are compiled at their first use",
           file=sys.stderr, flush=True)
     model = load_model(args.model, dtype=args.dtype)
-    engine = Engine(model, max_tokens=args.max_tokens)
+    engine = Engine(model, max_tokens=cache_tokens(args.max_tokens))
     print("[trace_run] ready", file=sys.stderr, flush=True)
     Replay(engine, args.out).run(sys.stdin)
     return 0

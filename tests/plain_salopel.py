@@ -156,3 +156,14 @@ def forward(ids, weights, config, dtype=torch.float64, layers_out=None):
             layers_out.append(x.clone())
     x = norm_around_zero(x, w["final.norm"], eps)
     return x @ w["embed"].T
+
+
+def greedy(ids, weights, config, steps, dtype=torch.float64):
+    """Greedy continuation: the whole sequence is recomputed for every new token; ties go to the
+    lowest index."""
+    ids, out = list(ids), []
+    for _ in range(steps):
+        token = int(torch.argmax(forward(ids, weights, config, dtype)[-1]))
+        out.append(token)
+        ids.append(token)
+    return out
