@@ -1,7 +1,7 @@
 """Throughput of GPT-2 generation on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 48] [--dtype bf16]
-                    [--repetitions 10] [--workload xl|small|medium|sweep] [--model xl|medium|small]
+                    [--repetitions 10] [--workload xl|small|medium|sweep|salopel] [--model xl|medium|small]
                     [--kernel-batches 1,64] [--sweep-part all|decode|prompts] [--no-points] [--no-kernels] [--no-own]
 
 The default workload (``xl``) has the layer sizes of GPT-2 XL with random weights: a batch of 8
@@ -44,6 +44,9 @@ generation loop: GPT-2 small sizes in float32, 16 prompts of 1 to 1,000 tokens d
 and sampled at temperature 1 to 1,024 tokens each.  Their value is generated tokens per second.
 ``--workload sweep`` prints a table of further sizes (decode over batch sizes and contexts up to
 8,192 tokens, prompts of 64 to 8,192 tokens whole and in chunks of 256) instead of the JSON line.
+``--workload salopel`` runs the library's second family, Salopel, at two widths whose layers resemble
+a real model's, beside GPT-2 at equal width, depth, feed-forward and vocabulary: prompt and decode
+throughput and each model's classes of kernels, one JSON line per width.
 """
 
 import argparse
@@ -192,6 +195,35 @@ def _class_of(name, call):
         return f"embed {call.tokens}x{call.width}", call.tokens * call.width * 6, 0.0
     if short == "kv_copy":
         return f"kv_copy {call.tokens}tok", call.tokens * call.kv.kv_heads * call.kv.head_dim * 8, 0.0
+    if short == "output_norm":
+        return f"output_norm {call.tokens}x{call.width}", (call.n_delta + 2) * call.tokens * call.width * 4 + \
+            (call.tokens * call.cast_cols * 2 if call.cast else 0), 0.0
+    if short == "poly_norm":
+        return f"poly_norm {call.tokens}x{call.columns}", call.tokens * call.columns * 6, 0.0
+    if short == "latent_norm":
+        return f"latent_norm {call.tokens}tok", call.tokens * (call.q_rank + call.kv_rank) * 8, 0.0
+    if short == "head_project":
+        element = 4 if call.dtype == 0 else 2
+        work = call.heads * call.vdim * call.rank
+        return f"head_project {call.tokens}x{call.heads}x{call.vdim}x{call.rank}", \
+            work * element + call.tokens * call.heads * (call.rank + call.vdim) * element + call.tokens * call.heads * call.vdim * 4, \
+            2.0 * call.tokens * work
+    if short == "causal_conv":
+        return f"causal_conv {call.tokens}x{call.channels}", call.tokens * call.channels * 8 + call.n_seqs * call.taps * call.channels * 8, 0.0
+    if short == "dt_project":
+        return f"dt_project {call.tokens}x{call.channels}x{call.rank}", call.channels * call.rank * 2 + call.tokens * (call.channels + call.rank) * 4, \
+            2.0 * call.tokens * call.channels * call.rank
+    if short == "selective_scan":       # state read and written, five values a token and channel, B and C
+        return f"selective_scan {call.tokens}x{call.channels}x{call.state}", \
+            call.n_seqs * call.channels * call.state * 8 + call.tokens * (call.channels * 14 + call.state * 8) + call.channels * call.state * 4, \
+            6.0 * call.tokens * call.channels * call.state
+    if short == "head_scan":
+        inner = call.heads * call.vdim
+        return f"head_scan {call.tokens}x{call.heads}x{call.vdim}x{call.state}", \
+            call.n_seqs * inner * call.state * 8 + call.tokens * (inner * 8 + call.groups * call.state * 8), \
+            6.0 * call.tokens * inner * call.state
+    if short == "gated_norm":
+        return f"gated_norm {call.tokens}x{call.channels}", call.tokens * call.channels * 10, 0.0
     return short, 0, 0.0
 
 
@@ -474,6 +506,89 @@ def run_sweep(args):
             print(f"prompt\t{tokens}\t{chunk}\t{seconds * 1e3:.3f}\t{tokens / seconds:.0f}\t{flops / seconds / PEAK_FLOPS[dtype]:.3f}", flush=True)
 
 
+# --- a second family beside GPT-2 at equal sizes ------------------------------------------------
+
+def salopel_config(width, layers, vocab):
+    """Salopel at layer sizes that resemble a real model's: groups of four layers (latent attention
+    with a feed-forward, a scan with one decay per head, a selective scan, latent attention with a
+    feed-forward), heads of 64 and 128, a latent of 128 for keys and values, inner widths of 2 x width
+    in the recurrent layers and 4 x width in the feed-forward."""
+    heads = min(16, width // 64)
+    attention = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": 4 * width},
+                 "mixer": {"heads": heads, "dim": 128, "vdim": 64, "q_rank": 3 * width // 8 // 8 * 8, "kv_rank": 128,
+                           "scale": 128 ** -0.5}}
+    per_head = {"type": "mamba2", "mlp": None,
+                "mixer": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 1, "norm_groups": 1, "conv": 4}}
+    per_channel = {"type": "mamba1", "mlp": None,
+                   "mixer": {"inner": 2 * width, "state": 16, "dt_rank": width // 16, "conv": 4}}
+    group = [attention, per_head, per_channel, attention]
+    return {"architecture": "Salopel", "vocab": vocab, "width": width, "residual_mult": 0.5, "norm": {"eps": 1e-5},
+            "layers": [dict(group[i % 4]) for i in range(layers)]}
+
+
+def build_salopel(config, dtype):
+    import torch
+
+    import burn_transformers_amd as bt
+    family = bt.resolve_family(config)
+    tensors = family.init(family.config_class.from_dict(config), torch.Generator().manual_seed(0))
+    return bt.model_from_tensors(config, {k: v.to(torch.bfloat16) for k, v in tensors.items()},
+                                 dtype="bfloat16" if dtype == "bf16" else "float32")
+
+
+def run_salopel(args):
+    """Prompt and decode throughput of Salopel beside GPT-2 at equal width, depth, feed-forward and
+    vocabulary, with each model's classes of kernels on their own.  One JSON line per width."""
+    import torch
+
+    import burn_transformers_amd as bt
+    dtype = args.dtype or "bf16"
+    layers, batch, prompt_len, steps = args.layers or 12, args.batch, 512, min(args.steps, 64)
+    vocab = 32000
+    for width in (1024, 2048):
+        line = {"workload": "salopel beside gpt2", "width": width, "layers": layers, "dtype": dtype, "batch": batch,
+                "prompt_len": prompt_len, "decode_steps": steps, "data": "synthetic token ids, random weights"}
+        for name in ("salopel", "gpt2"):
+            if name == "salopel":
+                config = salopel_config(width, layers, vocab)
+                model = build_salopel(config, dtype)
+            else:
+                config = dict(XL, n_layer=layers, n_embd=width, n_head=width // 64, n_inner=4 * width, vocab_size=vocab,
+                              n_positions=2048)
+                model = build_model(config, dtype)
+            engine = bt.Engine(model, max_tokens=max(batch, 8) * 2048)
+            times, done, _ = decode_run(engine, batch, 8, steps, vocab, max(3, args.repetitions // 2), 1, prompt_len=prompt_len)
+            decode_seconds = statistics.median(times) / done
+            prefill_seconds = statistics.median(prefill_run(engine, vocab, max(3, args.repetitions // 2)))
+            result = {"decode_tokens_per_s": round(batch / decode_seconds, 1), "decode_ms_per_step": round(decode_seconds * 1e3, 4),
+                      "prefill_tokens_per_s": round(PREFILL_SEQS * PREFILL_LEN / prefill_seconds, 1),
+                      "prefill_ms": round(prefill_seconds * 1e3, 3),
+                      "parameters": sum(t.numel() for t in model.store.values())}
+            if not args.no_kernels:
+                context = prompt_len + steps // 2
+                prompts = synthetic_prompts(batch, context - 1, vocab, seed=7)
+                slots = [engine.open() for _ in prompts]
+                engine.step(list(zip(slots, prompts)))
+                kv = batch * context * 2 * 128 * ELEMENT_BYTES[dtype] if name == "salopel" else batch * context * 2 * width * ELEMENT_BYTES[dtype]
+                flops = 4.0 * batch * context * (128 * min(16, width // 64) if name == "salopel" else width)
+                result["decode_kernels"] = kernel_classes(engine, [(slot, [5]) for slot in slots], kv, flops, PEAK_FLOPS[dtype])
+                for slot in slots:
+                    engine.close(slot)
+                prompts = synthetic_prompts(PREFILL_SEQS, PREFILL_LEN, vocab, seed=8)
+                slots = [engine.open() for _ in prompts]
+                tokens = PREFILL_SEQS * PREFILL_LEN
+                per_token = 128 * min(16, width // 64) if name == "salopel" else width
+                result["prefill_kernels"] = kernel_classes(engine, list(zip(slots, prompts)), 4 * tokens * per_token * ELEMENT_BYTES[dtype],
+                                                           PREFILL_SEQS * 2.0 * per_token * PREFILL_LEN * (PREFILL_LEN + 1),
+                                                           PEAK_FLOPS[dtype], replays=10)
+                for slot in slots:
+                    engine.close(slot)
+            line[name] = result
+            del engine, model
+            torch.cuda.empty_cache()
+        print(json.dumps(line), flush=True)
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -486,7 +601,7 @@ def main():
     parser.add_argument("--kernel-batches", default="", help="further batch sizes whose decode kernel classes are timed, e.g. 1,64")
     parser.add_argument("--dtype", choices=["bf16", "fp32"], default=None)
     parser.add_argument("--repetitions", type=int, default=10, help="measured repetitions, each on fresh sequences")
-    parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep"], default="xl")
+    parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep", "salopel"], default="xl")
     parser.add_argument("--sweep-part", choices=["all", "decode", "prompts"], default="all",
                         help="which table of --workload sweep to run")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
@@ -499,6 +614,9 @@ def main():
     if args.repetitions < 1:
         parser.error("--repetitions must be at least 1")
     args.kernel_batches = [int(b) for b in args.kernel_batches.split(",") if b]
+    if args.workload == "salopel":
+        run_salopel(args)
+        return
     if args.layers is None:
         args.layers = XL["n_layer"] if args.workload == "sweep" else MODELS[args.model]["n_layer"]
     if args.workload == "sweep":
