@@ -150,6 +150,32 @@ __global__ void __launch_bounds__(256) head_project_kernel(HeadProjectCall c) {
     }
 }
 
+// The same for steps of few tokens (decode): one work-group per (token, head, run of 64 outputs), four
+// lanes share an output and split the rank, everything read straight from memory with all loads of
+// a lane independent of each other.
+#define HP_SMALL_TOKENS 32
+
+template <typename T>
+__global__ void __launch_bounds__(256) head_project_small_kernel(HeadProjectCall c) {
+  const int t = blockIdx.x, head = blockIdx.y;
+  const int v = blockIdx.z * 64 + (threadIdx.x >> 2), part = threadIdx.x & 3;
+  const bool live = v < c.vdim;
+  const int col = head * c.vdim + (live ? v : c.vdim - 1);
+  const T* w = static_cast<const T*>(c.W) + (int64_t)col * c.rank;
+  const T* ctx = static_cast<const T*>(c.ctx) + (int64_t)t * c.ld_ctx + (int64_t)head * c.head_pitch;
+  float acc = 0.f;
+  for (int r = part; r < c.rank; r += 4) acc = fmaf(to_float(w[r]), to_float(ctx[r]), acc);
+  acc += __shfl_xor(acc, 2, 64);
+  acc += __shfl_xor(acc, 1, 64);
+  T* out = static_cast<T*>(c.out) + (int64_t)t * c.ld_out;
+  if (live && part == 0) {
+    if (c.gate) acc *= 1.0f / (1.0f + expf(-c.gate[(int64_t)t * c.ld_gate + col]));
+    out[col] = from_float<T>(acc);
+  }
+  if (head == c.heads - 1 && blockIdx.z == gridDim.z - 1)
+    for (int extra = c.heads * c.vdim + threadIdx.x; extra < c.out_cols; extra += 256) out[extra] = from_float<T>(0.f);
+}
+
 BT_EXPORT int bt_head_project_call(void* stream, const HeadProjectCall* c) {
   if (c->tokens <= 0) return BT_OK;
   if (c->heads <= 0 || c->vdim <= 0 || c->rank <= 0)
@@ -159,6 +185,14 @@ BT_EXPORT int bt_head_project_call(void* stream, const HeadProjectCall* c) {
       (c->gate && c->ld_gate < (int64_t)c->heads * c->vdim))
     BT_REFUSE("head_project: the rows do not hold %d heads", c->heads);
   if (!c->ctx || !c->W || !c->out) BT_REFUSE("head_project: missing operand");
+  if (c->tokens <= HP_SMALL_TOKENS) {
+    dim3 small(c->tokens, c->heads, (c->vdim + 63) / 64);
+    if (c->dtype == 0)
+      hipLaunchKernelGGL(head_project_small_kernel<float>, small, dim3(256), 0, (hipStream_t)stream, *c);
+    else
+      hipLaunchKernelGGL(head_project_small_kernel<bf16_t>, small, dim3(256), 0, (hipStream_t)stream, *c);
+    return bt_check_launch("head_project");
+  }
   dim3 grid((c->tokens + HP_TOKENS - 1) / HP_TOKENS, c->heads, (c->vdim + HP_VCHUNK - 1) / HP_VCHUNK), block(256);
   if (c->dtype == 0)
     hipLaunchKernelGGL(head_project_kernel<float>, grid, block, 0, (hipStream_t)stream, *c);

@@ -9,6 +9,29 @@
 //   * gate, then RMS norm in equal parts
 #include "host.h"
 
+#define FILL 16      // elements a lane brings into LDS at a time, with loads that are all in flight together
+
+// Sums over groups of 8 or 16 neighbouring lanes with data-parallel moves between lanes of a row
+// (no trip through the LDS crossbar as a shuffle takes; a recurrence pays this once per token): first
+// within quads (swap neighbours, swap pairs: then every lane of a quad holds the quad's sum), then
+// the mirror image within half a row pairs the two quads of eight lanes, then the mirror image within
+// the row pairs its halves.  Every lane of the group ends with the group's sum.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float sum_of_8_lanes(float v) {
+  v += dpp_move<0xB1>(v);     // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);     // quad_perm [2, 3, 0, 1]
+  v += dpp_move<0x141>(v);    // row_half_mirror
+  return v;
+}
+__device__ __forceinline__ float sum_of_16_lanes(float v) {
+  v = sum_of_8_lanes(v);
+  v += dpp_move<0x140>(v);    // row_mirror
+  return v;
+}
+
 __device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
 __device__ __forceinline__ float softplus_f(float v) { return v > 20.0f ? v : log1pf(expf(v)); }
 
@@ -156,8 +179,7 @@ BT_EXPORT int bt_dt_project_call(void* stream, const DtProjectCall* c) {
 //   S[c][n] <- exp(dt_c * A[c][n]) * S[c][n] + dt_c * x_c * B_n,   A = -exp(A_log)
 //   y_c = sum_n S[c][n] * C_n + D_c * x_c;   out_c = y_c * silu(z_c)
 // One wave per (8 channels, sequence): eight lanes share a channel, lane j of them owns the state
-// elements j, j + 8, ... in registers (R of them); a token's inputs are asked for U tokens at a time,
-// so that their latency is paid once per U tokens and not once per token.
+// elements j, j + 8, ... in registers (R of them).
 struct SelectiveScanCall {
   int out_dtype;
   int tokens, n_seqs, channels, state;
@@ -181,10 +203,19 @@ struct SelectiveScanCall {
   const int* slots;
 };
 
-template <typename T, int R, int U>
-__global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c) {
-  const int lane = threadIdx.x, sub = lane & 7;
-  const int ch = blockIdx.x * 8 + (lane >> 3), seq = blockIdx.y;
+// LDS holds a run of `chunk` tokens' inputs (B and C rows padded to 8 R with zeros, and the wave's eight
+// channels' dt, x and z), brought in with loads that are all in flight together: one round trip to
+// memory per run of tokens instead of one per token, which is what bounds a recurrence.
+template <typename T, int R>
+__global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c, int chunk) {
+  extern __shared__ float lds[];
+  constexpr int NP = 8 * R;
+  float2* BC = reinterpret_cast<float2*>(lds);   // [chunk][NP] pairs (B, C): one 8-byte read for both
+  float* dts = lds + (size_t)chunk * NP * 2;     // [chunk][8]
+  float* xs = dts + (size_t)chunk * 8;
+  float* zs = xs + (size_t)chunk * 8;
+  const int lane = threadIdx.x, sub = lane & 7, cl = lane >> 3;
+  const int ch = blockIdx.x * 8 + cl, seq = blockIdx.y;
   const bool live = ch < c.channels;
   const int chs = live ? ch : c.channels - 1;        // idle lanes read a valid channel and write nothing
   const int first = c.seq_off[seq], last = c.seq_off[seq + 1];
@@ -198,37 +229,60 @@ __global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c)
   }
   const float Dc = c.D[chs];
   T* out = static_cast<T*>(c.out);
-  for (int t0 = first; t0 < last; t0 += U) {
-    float dt[U], xv[U], zv[U], Bv[U][R], Cv[U][R];
+  for (int t0 = first; t0 < last; t0 += chunk) {
+    const int count = min(chunk, last - t0);
+    __syncthreads();
+    // (several elements of a lane at a time, all loads issued before the first is stored: a loop of
+    // single loads would wait for memory once per element)
+    for (int e0 = lane; e0 < count * NP; e0 += 64 * FILL) {
+      float2 held_bc[FILL];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int t = min(t0 + u, last - 1);
-      dt[u] = c.dt[(int64_t)t * c.ld_dt + chs];
-      xv[u] = c.x[(int64_t)t * c.ld_x + chs];
-      zv[u] = c.z[(int64_t)t * c.ld_z + chs];
+      for (int k = 0; k < FILL; ++k) {
+        const int e = e0 + 64 * k, i = e / NP, n = e % NP;
+        held_bc[k] = (e < count * NP && n < c.state)
+                         ? make_float2(c.B[(int64_t)(t0 + i) * c.ld_bc + n], c.C[(int64_t)(t0 + i) * c.ld_bc + n])
+                         : make_float2(0.f, 0.f);
+      }
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const int n = sub + 8 * r;
-        Bv[u][r] = n < c.state ? c.B[(int64_t)t * c.ld_bc + n] : 0.f;
-        Cv[u][r] = n < c.state ? c.C[(int64_t)t * c.ld_bc + n] : 0.f;
+      for (int k = 0; k < FILL; ++k)
+        if (e0 + 64 * k < count * NP) BC[e0 + 64 * k] = held_bc[k];
+    }
+    {
+      float held_in[8][3];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {          // count <= 64 tokens of 8 channels: at most eight elements a lane
+        const int e = lane + 64 * k, i = min(e >> 3, count - 1);
+        const int q = min((int)blockIdx.x * 8 + (e & 7), c.channels - 1);
+        held_in[k][0] = c.dt[(int64_t)(t0 + i) * c.ld_dt + q];
+        held_in[k][1] = c.x[(int64_t)(t0 + i) * c.ld_x + q];
+        held_in[k][2] = c.z[(int64_t)(t0 + i) * c.ld_z + q];
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int e = lane + 64 * k;
+        if (e < count * 8) {
+          dts[e] = held_in[k][0];
+          xs[e] = held_in[k][1];
+          zs[e] = held_in[k][2];
+        }
       }
     }
+    __syncthreads();
+    // (four tokens' reads from LDS and sums are in flight together; only the state ties them)
+#pragma unroll 4
+    for (int i = 0; i < count; ++i) {
+      const float dt = dts[i * 8 + cl], xv = xs[i * 8 + cl];
+      const float dx = dt * xv;
+      float acc = 0.f;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (t0 + u < last) {
-        const float dx = dt[u] * xv[u];
-        float acc = 0.f;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          S[r] = expf(dt[u] * A[r]) * S[r] + dx * Bv[u][r];
-          acc = fmaf(S[r], Cv[u][r], acc);
-        }
-        acc += __shfl_xor(acc, 4, 64);
-        acc += __shfl_xor(acc, 2, 64);
-        acc += __shfl_xor(acc, 1, 64);
-        if (live && sub == 0)
-          out[(int64_t)(t0 + u) * c.ld_out + ch] = from_float<T>((acc + Dc * xv[u]) * silu_f(zv[u]));
+      for (int r = 0; r < R; ++r) {
+        const float2 bc = BC[i * NP + sub + 8 * r];
+        S[r] = expf(dt * A[r]) * S[r] + dx * bc.x;
+        acc = fmaf(S[r], bc.y, acc);
       }
+      acc = sum_of_8_lanes(acc);
+      if (live && sub == 0)
+        out[(int64_t)(t0 + i) * c.ld_out + ch] = from_float<T>((acc + Dc * xv) * silu_f(zs[i * 8 + cl]));
     }
   }
   if (live) {
@@ -244,16 +298,30 @@ __global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c)
       for (int col = c.channels + lane; col < c.out_cols; col += 64) out[(int64_t)t * c.ld_out + col] = from_float<T>(0.f);
 }
 
+// Tokens of a run: as many as keep a work-group's LDS at about 24 KiB, at most 64, no more than the step has.
+static int scan_chunk(int floats_per_token, int tokens) {
+  int chunk = 6144 / floats_per_token;
+  chunk = chunk < 1 ? 1 : chunk > 64 ? 64 : chunk;
+  return chunk < tokens ? chunk : tokens;
+}
+
+template <typename T, int R>
+static void launch_selective_scan_r(hipStream_t stream, const SelectiveScanCall& c) {
+  const int per_token = 2 * 8 * R + 24;
+  const int chunk = scan_chunk(per_token, c.tokens);
+  dim3 grid((c.channels + 7) / 8, c.n_seqs), block(64);
+  hipLaunchKernelGGL((selective_scan_kernel<T, R>), grid, block, (size_t)chunk * per_token * sizeof(float), stream, c, chunk);
+}
+
 template <typename T>
 static int launch_selective_scan(hipStream_t stream, const SelectiveScanCall& c) {
-  dim3 grid((c.channels + 7) / 8, c.n_seqs), block(64);
   const int per = (c.state + 7) / 8;
-  if (per <= 1) hipLaunchKernelGGL((selective_scan_kernel<T, 1, 8>), grid, block, 0, stream, c);
-  else if (per <= 2) hipLaunchKernelGGL((selective_scan_kernel<T, 2, 8>), grid, block, 0, stream, c);
-  else if (per <= 4) hipLaunchKernelGGL((selective_scan_kernel<T, 4, 4>), grid, block, 0, stream, c);
-  else if (per <= 8) hipLaunchKernelGGL((selective_scan_kernel<T, 8, 2>), grid, block, 0, stream, c);
-  else if (per <= 16) hipLaunchKernelGGL((selective_scan_kernel<T, 16, 1>), grid, block, 0, stream, c);
-  else hipLaunchKernelGGL((selective_scan_kernel<T, 32, 1>), grid, block, 0, stream, c);
+  if (per <= 1) launch_selective_scan_r<T, 1>(stream, c);
+  else if (per <= 2) launch_selective_scan_r<T, 2>(stream, c);
+  else if (per <= 4) launch_selective_scan_r<T, 4>(stream, c);
+  else if (per <= 8) launch_selective_scan_r<T, 8>(stream, c);
+  else if (per <= 16) launch_selective_scan_r<T, 16>(stream, c);
+  else launch_selective_scan_r<T, 32>(stream, c);
   return bt_check_launch("selective_scan");
 }
 
@@ -289,71 +357,95 @@ struct HeadScanCall {
   const float* D;         // [heads]
   float* y;               // [tokens][ld_y] float32: head h at columns h * vdim
   int64_t ld_y;
-  float* S;               // slot s: [heads][state][vdim] at S + s * state_stride
+  float* S;               // slot s: [heads][vdim / 4 rounded up][state][4] at S + s * state_stride
   int64_t state_stride;
   const int* seq_off;
   const int* slots;
 };
 
-template <int R, int U>
-__global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c) {
-  const int lane = threadIdx.x, sub = lane & 15;
-  const int p = blockIdx.x * 4 + (lane >> 4), head = blockIdx.y, seq = blockIdx.z;
+// The state of a slot is laid out for this kernel's lanes: [heads][tiles of 4 channels][state][4], so
+// that a wave's load of one register's worth of state (16 state elements by 4 channels) is 256
+// contiguous bytes.  Nobody else reads it; a new sequence's state is all zeros in any layout.
+template <int R>
+__global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk) {
+  extern __shared__ float lds[];
+  constexpr int NP = 16 * R;
+  float2* BC = reinterpret_cast<float2*>(lds);   // [chunk][NP] pairs (B, C): one 8-byte read for both
+  float* xs = lds + (size_t)chunk * NP * 2;      // [chunk][4]
+  float* steps = xs + (size_t)chunk * 4;   // [chunk] dt after bias and softplus
+  float* decays = steps + chunk;           // [chunk]
+  const int lane = threadIdx.x, sub = lane & 15, pl = lane >> 4;
+  const int tile = blockIdx.x, tiles = gridDim.x, head = blockIdx.y, seq = blockIdx.z;
+  const int p = tile * 4 + pl;
   const bool live = p < c.vdim;
-  const int ps = live ? p : c.vdim - 1;
   const int group = head / (c.heads / c.groups);
   const int first = c.seq_off[seq], last = c.seq_off[seq + 1];
-  float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + (int64_t)head * c.state * c.vdim + ps;
+  float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + ((int64_t)head * tiles + tile) * c.state * 4 + pl;
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int n = sub + 16 * r;
-    S[r] = n < c.state ? held[(int64_t)n * c.vdim] : 0.f;
+    S[r] = n < c.state ? held[(int64_t)n * 4] : 0.f;
   }
   const float rate = -expf(c.A_log[head]), bias = c.dt_bias[head], Dh = c.D[head];
-  const float* xcol = c.x + head * c.vdim + ps;
   const float* Bg = c.B + group * c.state;
   const float* Cg = c.C + group * c.state;
-  for (int t0 = first; t0 < last; t0 += U) {
-    float dt[U], xv[U], Bv[U][R], Cv[U][R];
+  for (int t0 = first; t0 < last; t0 += chunk) {
+    const int count = min(chunk, last - t0);
+    __syncthreads();
+    // (sixteen elements of a lane at a time, all loads issued before the first is stored: a loop of
+    // single loads would wait for memory once per element)
+    for (int e0 = lane; e0 < count * NP; e0 += 64 * FILL) {
+      float2 held_bc[FILL];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int t = min(t0 + u, last - 1);
-      dt[u] = c.dt_raw[(int64_t)t * c.ld_dt + head];
-      xv[u] = xcol[(int64_t)t * c.ld];
+      for (int k = 0; k < FILL; ++k) {
+        const int e = e0 + 64 * k, i = e / NP, n = e % NP;
+        held_bc[k] = (e < count * NP && n < c.state)
+                         ? make_float2(Bg[(int64_t)(t0 + i) * c.ld + n], Cg[(int64_t)(t0 + i) * c.ld + n]) : make_float2(0.f, 0.f);
+      }
+#pragma unroll
+      for (int k = 0; k < FILL; ++k)
+        if (e0 + 64 * k < count * NP) BC[e0 + 64 * k] = held_bc[k];
+    }
+    for (int e = lane; e < count * 4; e += 64) {
+      const int i = e >> 2, q = tile * 4 + (e & 3);
+      xs[e] = q < c.vdim ? c.x[(int64_t)(t0 + i) * c.ld + head * c.vdim + q] : 0.f;
+    }
+    for (int e = lane; e < count; e += 64) {
+      const float step = softplus_f(c.dt_raw[(int64_t)(t0 + e) * c.ld_dt + head] + bias);
+      steps[e] = step;
+      decays[e] = expf(rate * step);
+    }
+    __syncthreads();
+    // (four tokens' reads from LDS and sums are in flight together; only the state ties them)
+#pragma unroll 4
+    for (int i = 0; i < count; ++i) {
+      const float xv = xs[i * 4 + pl], decay = decays[i];
+      const float dx = steps[i] * xv;
+      float acc = 0.f;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const int n = sub + 16 * r;
-        Bv[u][r] = n < c.state ? Bg[(int64_t)t * c.ld + n] : 0.f;
-        Cv[u][r] = n < c.state ? Cg[(int64_t)t * c.ld + n] : 0.f;
+        const float2 bc = BC[i * NP + sub + 16 * r];
+        S[r] = decay * S[r] + dx * bc.x;
+        acc = fmaf(S[r], bc.y, acc);
       }
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (t0 + u < last) {
-        const float step = softplus_f(dt[u] + bias);
-        const float decay = expf(rate * step), dx = step * xv[u];
-        float acc = 0.f;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          S[r] = decay * S[r] + dx * Bv[u][r];
-          acc = fmaf(S[r], Cv[u][r], acc);
-        }
-        acc += __shfl_xor(acc, 8, 64);
-        acc += __shfl_xor(acc, 4, 64);
-        acc += __shfl_xor(acc, 2, 64);
-        acc += __shfl_xor(acc, 1, 64);
-        if (live && sub == 0) c.y[(int64_t)(t0 + u) * c.ld_y + head * c.vdim + p] = acc + Dh * xv[u];
-      }
+      acc = sum_of_16_lanes(acc);
+      if (live && sub == 0) c.y[(int64_t)(t0 + i) * c.ld_y + head * c.vdim + p] = acc + Dh * xv;
     }
   }
-  if (live) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int n = sub + 16 * r;
-      if (n < c.state) held[(int64_t)n * c.vdim] = S[r];
-    }
+  for (int r = 0; r < R; ++r) {
+    const int n = sub + 16 * r;
+    if (n < c.state) held[(int64_t)n * 4] = S[r];
   }
+}
+
+template <int R>
+static void launch_head_scan_r(hipStream_t stream, const HeadScanCall& c) {
+  const int per_token = 2 * 16 * R + 6;
+  const int chunk = scan_chunk(per_token, c.tokens);
+  dim3 grid((c.vdim + 3) / 4, c.heads, c.n_seqs), block(64);
+  hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, (size_t)chunk * per_token * sizeof(float), stream, c, chunk);
 }
 
 BT_EXPORT int bt_head_scan_call(void* stream, const HeadScanCall* c) {
@@ -363,16 +455,15 @@ BT_EXPORT int bt_head_scan_call(void* stream, const HeadScanCall* c) {
   if (!c->x || !c->B || !c->C || !c->dt_raw || !c->dt_bias || !c->A_log || !c->D || !c->y || !c->S || !c->seq_off || !c->slots)
     BT_REFUSE("head_scan: missing operand");
   if (c->ld_dt < c->heads || c->ld_y < (int64_t)c->heads * c->vdim ||
-      c->state_stride < (int64_t)c->heads * c->state * c->vdim)
+      c->state_stride < (int64_t)c->heads * c->state * ((c->vdim + 3) / 4 * 4))
     BT_REFUSE("head_scan: rows or state too short for %d heads of %d", c->heads, c->vdim);
-  dim3 grid((c->vdim + 3) / 4, c->heads, c->n_seqs), block(64);
   hipStream_t s = (hipStream_t)stream;
   const int per = (c->state + 15) / 16;
-  if (per <= 1) hipLaunchKernelGGL((head_scan_kernel<1, 8>), grid, block, 0, s, *c);
-  else if (per <= 2) hipLaunchKernelGGL((head_scan_kernel<2, 8>), grid, block, 0, s, *c);
-  else if (per <= 4) hipLaunchKernelGGL((head_scan_kernel<4, 4>), grid, block, 0, s, *c);
-  else if (per <= 8) hipLaunchKernelGGL((head_scan_kernel<8, 2>), grid, block, 0, s, *c);
-  else hipLaunchKernelGGL((head_scan_kernel<16, 1>), grid, block, 0, s, *c);
+  if (per <= 1) launch_head_scan_r<1>(s, *c);
+  else if (per <= 2) launch_head_scan_r<2>(s, *c);
+  else if (per <= 4) launch_head_scan_r<4>(s, *c);
+  else if (per <= 8) launch_head_scan_r<8>(s, *c);
+  else launch_head_scan_r<16>(s, *c);
   return bt_check_launch("head_scan");
 }
 

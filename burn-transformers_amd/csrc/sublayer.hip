@@ -56,6 +56,61 @@ __global__ void __launch_bounds__(256) output_norm_kernel(OutputNormCall c) {
       cast[(int64_t)t * c.ld_cast + col] = from_float<T>(0.f);
 }
 
+// The same for rows of up to 256 * KMAX columns: a thread's columns live in registers and every load
+// of a thread (partial sums, bias, the stream, the scale) is issued before the first is used, so a
+// row costs one round trip to memory.  A decode step has few rows: one row's latency is its time.
+template <typename T, int KMAX>
+__global__ void __launch_bounds__(256) output_norm_small_kernel(OutputNormCall c) {
+  __shared__ float scratch[32];
+  const int t = blockIdx.x;
+  float* xr = c.x + (int64_t)t * c.width;
+  float v[KMAX], xv[KMAX], g[KMAX];
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    const int col = threadIdx.x + 256 * k;
+    v[k] = xv[k] = g[k] = 0.f;
+    if (col < c.width) {
+      g[k] = c.gamma[col];
+      if (c.n_delta == 0) {
+        v[k] = xr[col];
+      } else {
+        if (c.accumulate) xv[k] = xr[col];
+        float sum = c.bias ? c.bias[col] : 0.f;
+        for (int s = 0; s < c.n_delta; ++s) sum += c.delta[s * c.delta_stride + (int64_t)t * c.ldd + col];
+        v[k] = sum;
+      }
+    }
+  }
+  float partial = 0.f;
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) partial += v[k] * v[k];
+  const float scale = c.mult / sqrtf(block_sum(partial, scratch) / (float)c.width + c.eps);
+  T* cast = static_cast<T*>(c.cast);
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    const int col = threadIdx.x + 256 * k;
+    if (col < c.width) {
+      const float y = v[k] * scale * g[k] + xv[k];
+      xr[col] = y;
+      if (cast) cast[(int64_t)t * c.ld_cast + col] = from_float<T>(y);
+    }
+  }
+  if (cast)
+    for (int col = c.width + threadIdx.x; col < c.cast_cols; col += blockDim.x)
+      cast[(int64_t)t * c.ld_cast + col] = from_float<T>(0.f);
+}
+
+template <typename T>
+static void launch_output_norm(hipStream_t stream, const OutputNormCall& c) {
+  dim3 grid(c.tokens), block(256);
+  if (c.width <= 1024)
+    hipLaunchKernelGGL((output_norm_small_kernel<T, 4>), grid, block, 0, stream, c);
+  else if (c.width <= 2048)
+    hipLaunchKernelGGL((output_norm_small_kernel<T, 8>), grid, block, 0, stream, c);
+  else
+    hipLaunchKernelGGL(output_norm_kernel<T>, grid, block, (size_t)c.width * sizeof(float), stream, c);
+}
+
 BT_EXPORT int bt_output_norm_call(void* stream, const OutputNormCall* c) {
   if (c->tokens <= 0) return BT_OK;
   if (c->width <= 0 || c->width > 15360) BT_REFUSE("output_norm: width %d outside 1..15360", c->width);
@@ -64,12 +119,10 @@ BT_EXPORT int bt_output_norm_call(void* stream, const OutputNormCall* c) {
   if (c->cast && (c->cast_cols < c->width || c->ld_cast < c->cast_cols))
     BT_REFUSE("output_norm: a copy of %d columns in rows of %lld does not hold width %d", c->cast_cols,
               (long long)c->ld_cast, c->width);
-  dim3 grid(c->tokens), block(256);
-  size_t lds = (size_t)c->width * sizeof(float);
   if (c->cast_dtype == 0)
-    hipLaunchKernelGGL(output_norm_kernel<float>, grid, block, lds, (hipStream_t)stream, *c);
+    launch_output_norm<float>((hipStream_t)stream, *c);
   else
-    hipLaunchKernelGGL(output_norm_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, *c);
+    launch_output_norm<bf16_t>((hipStream_t)stream, *c);
   return bt_check_launch("output_norm");
 }
 

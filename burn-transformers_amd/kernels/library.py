@@ -1068,7 +1068,8 @@ def selective_scan(x, z, dt, B, C, A_log, D, out, state, step):
 
 def head_scan(x, B, C, dt_raw, dt_bias, A_log, D, y, state, step, heads, vdim, elements, groups):
     """The scan with one decay per head (see csrc/state_space.hip); x, B and C are column ranges of
-    the same float32 rows; ``state`` [slots, >= heads * elements * vdim] float32."""
+    the same float32 rows; ``state`` [slots, >= heads * elements * vdim rounded up to 4] float32, in a
+    layout of the kernel's own."""
     if x.stride(0) != B.stride(0) or x.stride(0) != C.stride(0):
         raise KernelError("head_scan: x, B and C must be column ranges of the same rows")
     _launch(_module("state_space"), "bt_head_scan_call",

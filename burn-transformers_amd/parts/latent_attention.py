@@ -24,7 +24,7 @@ import torch
 from ..cache.storage import KVSpec
 from ..kernels import library as K
 from .attention import CausalSelfAttention
-from .base import Mixer, operand_columns, pad_columns, pad_rows
+from .base import Mixer, compute_units, operand_columns, pad_columns, pad_rows
 from .registry import register
 
 
@@ -88,11 +88,26 @@ class LatentAttention(Mixer):
                 names.append("attention_f32")
         return tuple(names)
 
-    # the planning of runs of keys is the ordinary attention's: one cached head, ``heads`` query heads
+    # the planning of a prompt's runs of keys is the ordinary attention's: one cached head, ``heads`` query heads
     kv_heads = 1
     window = 0
-    decode_runs = CausalSelfAttention.decode_runs
     prompt_runs = CausalSelfAttention.prompt_runs
+
+    def decode_runs(self, step, device):
+        """Into how many runs a decode step's keys are cut.  All heads share one cached head, so a
+        step has only as many work-groups as sequences unless the keys are cut, and they are cut much
+        earlier than where every head brings keys of its own: from ``SPLIT_BYTES`` of a sequence's
+        cached vectors on, into runs of at least ``RUN_BYTES``, as many as give every work-group a
+        compute unit.  Planned for the step's class of context, like the ordinary attention's."""
+        if not step.decode:
+            return 1
+        pair_bytes = step.context_limit * self.head_dim * 2 * (2 if step.dtype_is_bf16 else 4)
+        if pair_bytes <= self.SPLIT_BYTES:
+            return 1
+        return max(1, min(compute_units(device) // step.n_seqs, pair_bytes // self.RUN_BYTES, 64))
+
+    SPLIT_BYTES = 128 << 10
+    RUN_BYTES = 64 << 10
 
     def forward(self, h, step, memory, stream):
         tokens = h.shape[0]

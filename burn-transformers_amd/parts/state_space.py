@@ -119,7 +119,8 @@ class HeadScan(_Recurrent):
         self.out_weight = pad_columns(tensors["out_weight"], self.inner_cols)
         self.conv_weight, self.conv_bias = tensors["conv_weight"].contiguous(), tensors["conv_bias"]
         self.dt_bias, self.A_log, self.D, self.norm_weight = tensors["dt_bias"], tensors["A_log"], tensors["D"], tensors["norm_weight"]
-        self.conv_state, self.scan_state = (self.taps - 1) * self.channels, self.heads * self.state * self.vdim
+        # (the scan's kernel lays a head's state out in tiles of four channels)
+        self.conv_state, self.scan_state = (self.taps - 1) * self.channels, self.heads * self.state * ((self.vdim + 3) // 4 * 4)
 
     def forward(self, h, step, memory, stream):
         tokens, inner, bc = h.shape[0], self.inner, self.bc
