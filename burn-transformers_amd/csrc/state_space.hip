@@ -55,7 +55,9 @@ struct CausalConvCall {
   const int* slots;       // [n_seqs]
 };
 
-template <typename T>
+// SHIFT: every sequence of the step brings one token (a decode step), so a (sequence, channel) pair
+// belongs to one thread, which can also move the state on: no second kernel.
+template <typename T, bool SHIFT>
 __global__ void __launch_bounds__(256) causal_conv_kernel(CausalConvCall c) {
   const int t = blockIdx.x;
   const int ch = blockIdx.y * blockDim.x + threadIdx.x;
@@ -66,7 +68,7 @@ __global__ void __launch_bounds__(256) causal_conv_kernel(CausalConvCall c) {
   }
   const int seq = c.tok_seq[t];
   const int local = t - c.seq_off[seq];
-  const float* held = c.state + (int64_t)c.slots[seq] * c.state_stride;
+  float* held = c.state + (int64_t)c.slots[seq] * c.state_stride;
   float sum = c.bias[ch];
   for (int j = 0; j < c.taps; ++j) {
     const int back = c.taps - 1 - j;
@@ -78,6 +80,10 @@ __global__ void __launch_bounds__(256) causal_conv_kernel(CausalConvCall c) {
   const float y = silu_f(sum);
   c.out[(int64_t)t * c.ld_out + ch] = y;
   if (cast) cast[(int64_t)t * c.ld_cast + ch] = from_float<T>(y);
+  if (SHIFT) {
+    for (int r = 0; r + 2 < c.taps; ++r) held[(int64_t)r * c.channels + ch] = held[(int64_t)(r + 1) * c.channels + ch];
+    if (c.taps > 1) held[(int64_t)(c.taps - 2) * c.channels + ch] = c.in[(int64_t)t * c.ld_in + ch];
+  }
 }
 
 // After the convolution: the state becomes the last taps - 1 inputs of each sequence.
@@ -108,10 +114,17 @@ BT_EXPORT int bt_causal_conv_call(void* stream, const CausalConvCall* c) {
               (long long)c->state_stride, c->taps - 1, c->channels);
   const int cols = c->cast && c->cast_cols > c->channels ? c->cast_cols : c->channels;
   dim3 grid(c->tokens, (cols + 255) / 256), block(256);
+  if (c->tokens == c->n_seqs) {        // one token of every sequence
+    if (c->cast_dtype == 0)
+      hipLaunchKernelGGL((causal_conv_kernel<float, true>), grid, block, 0, (hipStream_t)stream, *c);
+    else
+      hipLaunchKernelGGL((causal_conv_kernel<bf16_t, true>), grid, block, 0, (hipStream_t)stream, *c);
+    return bt_check_launch("causal_conv");
+  }
   if (c->cast_dtype == 0)
-    hipLaunchKernelGGL(causal_conv_kernel<float>, grid, block, 0, (hipStream_t)stream, *c);
+    hipLaunchKernelGGL((causal_conv_kernel<float, false>), grid, block, 0, (hipStream_t)stream, *c);
   else
-    hipLaunchKernelGGL(causal_conv_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, *c);
+    hipLaunchKernelGGL((causal_conv_kernel<bf16_t, false>), grid, block, 0, (hipStream_t)stream, *c);
   int rc = bt_check_launch("causal_conv");
   if (rc || c->taps == 1) return rc;
   hipLaunchKernelGGL(conv_state_kernel, dim3(c->n_seqs, (c->channels + 255) / 256), block, 0, (hipStream_t)stream, *c);
@@ -131,13 +144,14 @@ struct DtProjectCall {
   int64_t ld_out;
 };
 
-#define DT_TOKENS 8
-
-template <typename T>
+// TOKENS tokens share a work-group (their rows of `low` wait in LDS, every weight is read once for
+// all of them); steps of few tokens take one token a work-group, which is more work-groups and a
+// shorter chain in each.
+template <typename T, int TOKENS>
 __global__ void __launch_bounds__(256) dt_project_kernel(DtProjectCall c) {
-  extern __shared__ float rows[];      // [DT_TOKENS][rank]
-  const int t0 = blockIdx.x * DT_TOKENS;
-  for (int e = threadIdx.x; e < DT_TOKENS * c.rank; e += blockDim.x) {
+  extern __shared__ float rows[];      // [TOKENS][rank]
+  const int t0 = blockIdx.x * TOKENS;
+  for (int e = threadIdx.x; e < TOKENS * c.rank; e += blockDim.x) {
     const int i = e / c.rank, r = e % c.rank;
     rows[e] = t0 + i < c.tokens ? c.low[(int64_t)(t0 + i) * c.ld_low + r] : 0.f;
   }
@@ -145,18 +159,25 @@ __global__ void __launch_bounds__(256) dt_project_kernel(DtProjectCall c) {
   const int ch = blockIdx.y * blockDim.x + threadIdx.x;
   if (ch >= c.channels) return;
   const T* w = static_cast<const T*>(c.W) + (int64_t)ch * c.rank;
-  float acc[DT_TOKENS];
+  float acc[TOKENS];
 #pragma unroll
-  for (int i = 0; i < DT_TOKENS; ++i) acc[i] = 0.f;
+  for (int i = 0; i < TOKENS; ++i) acc[i] = 0.f;
+#pragma unroll 8      // (eight of a thread's weights on their way at once)
   for (int r = 0; r < c.rank; ++r) {
     const float wv = to_float(w[r]);
 #pragma unroll
-    for (int i = 0; i < DT_TOKENS; ++i) acc[i] = fmaf(wv, rows[i * c.rank + r], acc[i]);
+    for (int i = 0; i < TOKENS; ++i) acc[i] = fmaf(wv, rows[i * c.rank + r], acc[i]);
   }
   const float b = c.bias[ch];
 #pragma unroll
-  for (int i = 0; i < DT_TOKENS; ++i)
+  for (int i = 0; i < TOKENS; ++i)
     if (t0 + i < c.tokens) c.out[(int64_t)(t0 + i) * c.ld_out + ch] = softplus_f(acc[i] + b);
+}
+
+template <typename T, int TOKENS>
+static void launch_dt_project(hipStream_t stream, const DtProjectCall& c) {
+  dim3 grid((c.tokens + TOKENS - 1) / TOKENS, (c.channels + 255) / 256), block(256);
+  hipLaunchKernelGGL((dt_project_kernel<T, TOKENS>), grid, block, (size_t)TOKENS * c.rank * sizeof(float), stream, c);
 }
 
 BT_EXPORT int bt_dt_project_call(void* stream, const DtProjectCall* c) {
@@ -165,12 +186,14 @@ BT_EXPORT int bt_dt_project_call(void* stream, const DtProjectCall* c) {
     BT_REFUSE("dt_project: %d channels from rank %d (1..1024)", c->channels, c->rank);
   if (!c->low || !c->W || !c->bias || !c->out || c->ld_low < c->rank || c->ld_out < c->channels)
     BT_REFUSE("dt_project: missing operand or rows too short");
-  dim3 grid((c->tokens + DT_TOKENS - 1) / DT_TOKENS, (c->channels + 255) / 256), block(256);
-  size_t lds = (size_t)DT_TOKENS * c->rank * sizeof(float);
-  if (c->dtype == 0)
-    hipLaunchKernelGGL(dt_project_kernel<float>, grid, block, lds, (hipStream_t)stream, *c);
-  else
-    hipLaunchKernelGGL(dt_project_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, *c);
+  hipStream_t s = (hipStream_t)stream;
+  if (c->tokens <= 16) {
+    if (c->dtype == 0) launch_dt_project<float, 1>(s, *c);
+    else launch_dt_project<bf16_t, 1>(s, *c);
+  } else {
+    if (c->dtype == 0) launch_dt_project<float, 8>(s, *c);
+    else launch_dt_project<bf16_t, 8>(s, *c);
+  }
   return bt_check_launch("dt_project");
 }
 
@@ -268,9 +291,7 @@ __global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c,
       }
     }
     __syncthreads();
-    // (four tokens' reads from LDS and sums are in flight together; only the state ties them)
-#pragma unroll 4
-    for (int i = 0; i < count; ++i) {
+    auto token = [&](int i) {
       const float dt = dts[i * 8 + cl], xv = xs[i * 8 + cl];
       const float dx = dt * xv;
       float acc = 0.f;
@@ -283,7 +304,16 @@ __global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c,
       acc = sum_of_8_lanes(acc);
       if (live && sub == 0)
         out[(int64_t)(t0 + i) * c.ld_out + ch] = from_float<T>((acc + Dc * xv) * silu_f(zs[i * 8 + cl]));
+    };
+    // four tokens at a time, written out: their reads from LDS, exponentials and sums are in flight
+    // together and only the state ties them (the lane sums keep the compiler from unrolling a loop
+    // whose length it does not know)
+    int i = 0;
+    for (; i + 4 <= count; i += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) token(i + u);
     }
+    for (; i < count; ++i) token(i);
   }
   if (live) {
 #pragma unroll
@@ -390,6 +420,7 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
   const float rate = -expf(c.A_log[head]), bias = c.dt_bias[head], Dh = c.D[head];
   const float* Bg = c.B + group * c.state;
   const float* Cg = c.C + group * c.state;
+  float* ycol = c.y + head * c.vdim + (live ? p : 0);
   for (int t0 = first; t0 < last; t0 += chunk) {
     const int count = min(chunk, last - t0);
     __syncthreads();
@@ -417,9 +448,7 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
       decays[e] = expf(rate * step);
     }
     __syncthreads();
-    // (four tokens' reads from LDS and sums are in flight together; only the state ties them)
-#pragma unroll 4
-    for (int i = 0; i < count; ++i) {
+    auto token = [&](int i) {
       const float xv = xs[i * 4 + pl], decay = decays[i];
       const float dx = steps[i] * xv;
       float acc = 0.f;
@@ -430,8 +459,15 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
         acc = fmaf(S[r], bc.y, acc);
       }
       acc = sum_of_16_lanes(acc);
-      if (live && sub == 0) c.y[(int64_t)(t0 + i) * c.ld_y + head * c.vdim + p] = acc + Dh * xv;
+      if (live && sub == 0) ycol[(int64_t)(t0 + i) * c.ld_y] = acc + Dh * xv;
+    };
+    // four tokens at a time, written out (see selective_scan_kernel)
+    int i = 0;
+    for (; i + 4 <= count; i += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) token(i + u);
     }
+    for (; i < count; ++i) token(i);
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {

@@ -139,10 +139,30 @@ struct PolyNormCall {
   int64_t ldo;
 };
 
+// Three block-wide sums with one meeting of the waves (blocks of up to 1024 threads).
+__device__ __forceinline__ void block_sum3(float& a, float& b, float& d, float* scratch) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  d = wave_sum(d);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = (blockDim.x + 63) >> 6;
+  if (lane == 0) {
+    scratch[wave * 3] = a;
+    scratch[wave * 3 + 1] = b;
+    scratch[wave * 3 + 2] = d;
+  }
+  __syncthreads();
+  a = b = d = 0.f;
+  for (int w = 0; w < waves; ++w) {
+    a += scratch[w * 3];
+    b += scratch[w * 3 + 1];
+    d += scratch[w * 3 + 2];
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) poly_norm_kernel(PolyNormCall c) {
   extern __shared__ float row_buf[];
-  __shared__ float scratch[32];
+  __shared__ float scratch[48];
   const int t = blockIdx.x;
   const float* zr = c.z + (int64_t)t * c.ldz;
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
@@ -154,9 +174,7 @@ __global__ void __launch_bounds__(256) poly_norm_kernel(PolyNormCall c) {
     s4 += v2 * v2;
     s6 += v2 * v2 * v2;
   }
-  s2 = block_sum(s2, scratch);
-  s4 = block_sum(s4, scratch);
-  s6 = block_sum(s6, scratch);
+  block_sum3(s2, s4, s6, scratch);
   const float n = (float)c.columns;
   const float a = c.coefficients[0] / sqrtf(s2 / n + c.eps);
   const float b = c.coefficients[1] / sqrtf(s4 / n + c.eps);

@@ -256,3 +256,24 @@ def test_folder_round_trip_and_trace_replay(tmp_path):
         rows = torch.from_numpy(np.fromfile(tmp_path / "out" / f"{t + 1}.f32", dtype="<f4").reshape(2, -1))
         check(rows, torch.stack([want_a[15 + t], want_b[4 + t]]), "float32", f"replayed step {t + 1}")
     assert not engine.cache.ledger.live_slots()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_contexts_in_portions_and_decoded(dtype):
+    """A prompt of 1,500 tokens whole, in portions of 256 (portions behind a long context cut their
+    keys into runs), and decoded at its end (decode steps of long contexts cut theirs too)."""
+    engine = engine_for("attention", dtype, max_tokens=4096)
+    ids = prompts_for("attention", [1500], seed=12)[0]
+    want = plain_logits("attention", ids)
+    places = [0, 63, 64, 1023, 1024, 1279, 1280, 1499]
+    slot = engine.open()
+    check(engine.step([(slot, ids)], want=[places]).clone(), want[places], dtype, "long prompt, whole")
+    engine.close(slot)
+    slot = engine.open()
+    rows = []
+    for begin in range(0, 1280, 256):
+        rows.append(engine.step([(slot, ids[begin:begin + 256])], want=[[0, 255]]).clone())
+    check(torch.cat(rows), want[[p for b in range(0, 1280, 256) for p in (b, b + 255)]], dtype, "long prompt, in portions")
+    rows = [engine.step([(slot, [token])]).clone() for token in ids[1280:1300]]
+    check(torch.cat(rows), want[1280:1300], dtype, "long context, decoded")
+    engine.close(slot)
