@@ -24,7 +24,7 @@ import torch
 from ..cache.storage import KVSpec
 from ..kernels import library as K
 from .attention import CausalSelfAttention
-from .base import Mixer, compute_units, operand_columns, pad_columns, pad_rows
+from .base import Mixer, compute_units, operand_columns, packed_for_stream, pad_columns, pad_rows
 from .registry import register
 
 
@@ -75,6 +75,11 @@ class LatentAttention(Mixer):
         self.mixed_cols = operand_columns(self.heads * self.vdim, dtype)
         self.out_weight = pad_columns(tensors["out_weight"], self.mixed_cols)
         self.n_q = self.heads * self.head_dim
+        # second copies for decode steps, which read the weights and little else
+        on_gpu = self.fused_weight.is_cuda
+        self.fused_packed = K.PackedWeight(self.fused_weight) if on_gpu else None
+        self.query_packed = K.PackedWeight(self.query_weight) if on_gpu else None
+        self.out_packed = packed_for_stream(self.out_weight) if on_gpu else None
 
     def kv_spec(self):
         return KVSpec(1, self.head_dim, 0)
@@ -113,14 +118,14 @@ class LatentAttention(Mixer):
         tokens = h.shape[0]
         kv = memory.kv()
         fused = step.buffer("latent.fused", tokens, self.fused_cols, "float32")
-        K.gemm(h, self.fused_weight, K.epilogue_f32(fused))
+        K.gemm(h, self.fused_weight, K.epilogue_f32(fused), packed=self.fused_packed)
         c_q = step.buffer("latent.query_latent", tokens, self.q_cols, step.dtype)
         if not memory.writes:
             raise ValueError("latent attention: every run keeps a cache entry of its own")
         K.latent_norm(fused, self.q_rank, self.kv_offset, self.kv_rank, self.q_norm, self.kv_norm, self.eps, c_q,
                       step.tok_seq, step.tok_pos, kv, step.dtype)
         q = step.buffer("latent.queries", tokens, self.n_q, step.dtype)
-        K.gemm(c_q, self.query_weight, K.epilogue_store(q))
+        K.gemm(c_q, self.query_weight, K.epilogue_store(q), packed=self.query_packed)
         ctx = step.buffer("latent.context", tokens, self.n_q, step.dtype)
         partial, runs, prompt_runs = None, self.decode_runs(step, h.device), self.prompt_runs(step, h.device)
         if self.plain_only:
@@ -136,4 +141,4 @@ class LatentAttention(Mixer):
         mixed = step.buffer("latent.mixed", tokens, self.mixed_cols, step.dtype)
         K.head_project(ctx, self.up_v, self.heads, self.vdim, self.kv_rank, self.head_dim, mixed,
                        gate=fused[:, self.gate_offset:])
-        stream.add_product(step, mixed, self.out_weight)
+        stream.add_product(step, mixed, self.out_weight, packed=self.out_packed)

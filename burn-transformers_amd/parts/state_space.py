@@ -28,7 +28,7 @@ import torch
 
 from ..cache.storage import StateSpec
 from ..kernels import library as K
-from .base import Mixer, operand_columns, pad_columns
+from .base import Mixer, operand_columns, packed_for_stream, pad_columns
 from .registry import register
 
 
@@ -72,24 +72,29 @@ class SelectiveScan(_Recurrent):
         self.conv_weight, self.conv_bias = tensors["conv_weight"].contiguous(), tensors["conv_bias"]
         self.dt_bias, self.A_log, self.D = tensors["dt_bias"], tensors["A_log"].contiguous(), tensors["D"]
         self.conv_state, self.scan_state = (self.taps - 1) * self.inner, self.inner * self.state
+        # second copies for decode steps, which read the weights and little else
+        on_gpu = self.in_weight.is_cuda
+        self.in_packed = K.PackedWeight(self.in_weight) if on_gpu else None
+        self.x_packed = K.PackedWeight(self.x_weight) if on_gpu else None
+        self.out_packed = packed_for_stream(self.out_weight) if on_gpu else None
 
     def forward(self, h, step, memory, stream):
         tokens, inner = h.shape[0], self.inner
         conv_state, scan_state = self._state(memory)
         xz = step.buffer("scan.in", tokens, 2 * inner, "float32")
-        K.gemm(h, self.in_weight, K.epilogue_f32(xz))
+        K.gemm(h, self.in_weight, K.epilogue_f32(xz), packed=self.in_packed)
         x = step.buffer("scan.x", tokens, inner, "float32")
         # the next product reads x in the products' type; in a float32 model that is x itself
         cast = step.buffer("scan.x_operand", tokens, self.inner_cols, step.dtype) if step.dtype_is_bf16 else None
         K.causal_conv(xz[:, :inner], self.conv_weight, self.conv_bias, x, conv_state, step, cast=cast)
         low = step.buffer("scan.low", tokens, self.dt_rank + 2 * self.state, "float32")
-        K.gemm(cast if cast is not None else x, self.x_weight, K.epilogue_f32(low))
+        K.gemm(cast if cast is not None else x, self.x_weight, K.epilogue_f32(low), packed=self.x_packed)
         dt = step.buffer("scan.dt", tokens, inner, "float32")
         K.dt_project(low[:, :self.dt_rank], self.dt_weight, self.dt_bias, dt)
         gated = step.buffer("scan.gated", tokens, self.inner_cols, step.dtype)
         K.selective_scan(x, xz[:, inner:], dt, low[:, self.dt_rank:self.dt_rank + self.state],
                          low[:, self.dt_rank + self.state:], self.A_log, self.D, gated, scan_state, step)
-        stream.add_product(step, gated, self.out_weight)
+        stream.add_product(step, gated, self.out_weight, packed=self.out_packed)
 
 
 @register("mixer", "head_scan")
@@ -121,12 +126,15 @@ class HeadScan(_Recurrent):
         self.dt_bias, self.A_log, self.D, self.norm_weight = tensors["dt_bias"], tensors["A_log"], tensors["D"], tensors["norm_weight"]
         # (the scan's kernel lays a head's state out in tiles of four channels)
         self.conv_state, self.scan_state = (self.taps - 1) * self.channels, self.heads * self.state * ((self.vdim + 3) // 4 * 4)
+        on_gpu = self.in_weight.is_cuda
+        self.in_packed = K.PackedWeight(self.in_weight) if on_gpu else None
+        self.out_packed = packed_for_stream(self.out_weight) if on_gpu else None
 
     def forward(self, h, step, memory, stream):
         tokens, inner, bc = h.shape[0], self.inner, self.bc
         conv_state, scan_state = self._state(memory)
         fused = step.buffer("scan.in", tokens, inner + self.channels + self.heads, "float32")
-        K.gemm(h, self.in_weight, K.epilogue_f32(fused))
+        K.gemm(h, self.in_weight, K.epilogue_f32(fused), packed=self.in_packed)
         xbc = step.buffer("scan.x", tokens, self.channels, "float32")
         K.causal_conv(fused[:, inner:inner + self.channels], self.conv_weight, self.conv_bias, xbc, conv_state, step)
         y = step.buffer("scan.y", tokens, inner, "float32")
@@ -134,4 +142,4 @@ class HeadScan(_Recurrent):
                     self.dt_bias, self.A_log, self.D, y, scan_state, step, self.heads, self.vdim, self.state, self.groups)
         gated = step.buffer("scan.gated", tokens, self.inner_cols, step.dtype)
         K.gated_norm(y, fused[:, :inner], self.norm_weight, self.norm_groups, self.eps, gated)
-        stream.add_product(step, gated, self.out_weight)
+        stream.add_product(step, gated, self.out_weight, packed=self.out_packed)

@@ -277,3 +277,21 @@ def test_long_contexts_in_portions_and_decoded(dtype):
     rows = [engine.step([(slot, [token])]).clone() for token in ids[1280:1300]]
     check(torch.cat(rows), want[1280:1300], dtype, "long context, decoded")
     engine.close(slot)
+
+
+def test_command_line(capsys, tmp_path):
+    """The command line takes the family by config.json: random weights written from a configuration,
+    then greedy tokens for two prompts."""
+    import json
+    from burn_transformers_amd.cli import main
+    config, seed = CONFIGS["mixed"]
+    cfg_path = tmp_path / "cfg.json"
+    cfg_path.write_text(json.dumps(config))
+    prompts = prompts_for("mixed", [6, 13], seed=60)
+    text = ";".join(",".join(str(t) for t in p) for p in prompts)
+    assert main([str(tmp_path / "made"), text, "5", "--dtype", "float32", "--json", "--random-weights", str(cfg_path),
+                 "--weights-seed", str(seed)]) == 0
+    lines = [json.loads(line) for line in capsys.readouterr().out.strip().splitlines()]
+    weights = weights_for("mixed")
+    assert [line["token_ids"] for line in lines] == [plain.greedy(p, weights, config, 5) for p in prompts]
+    assert main([str(tmp_path / "made"), text, "4", "--temperature", "0.7", "--seed", "5", "--prefill-chunk-size", "4"]) == 0
