@@ -60,6 +60,10 @@ class NormalizedTokenEmbedding(Embedding):
         self.scale = (tensors["norm_weight"].float() + float(params.get("offset", 0.0))).contiguous()
         if tuple(self.token_table.shape) != (self.vocab_size, self.width) or tuple(self.scale.shape) != (self.width,):
             raise ValueError("embedding: table or scale do not have the configured sizes")
+        if self.token_table.dtype != self.scale.dtype and self.width % 8 != 0:
+            # the layers multiply by the stream's bfloat16 copy, whose rows the MFMA kernels read 16 bytes at a time
+            raise ValueError(f"embedding: the bfloat16 kernels take widths that are multiples of 8, not {self.width}; "
+                             f"load the model with dtype float32, which takes any width")
 
     def embed(self, step):
         x = step.buffer("stream.x", step.n_tokens, self.width, "float32")

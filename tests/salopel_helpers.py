@@ -59,7 +59,9 @@ ATTENTION_ONLY = model_config([latent(4, 32, 16, 24, 64, 0.25), latent(2, 16, 48
 SCAN_ONLY = model_config([mamba1(64, 16, 4, 3)], width=32, vocab=101, mult=0.7)
 HEADS_ONLY = model_config([mamba2(4, 16, 32, 2, 2, 4)], width=32, vocab=101, mult=0.7)
 FEED_FORWARD = model_config([latent(1, 8, 8, 8, 16, 1.0, ff=40)], width=32, vocab=61, mult=2.0)
-CONFIGS = {"mixed": (MIXED, 1), "odd": (ODD, 2), "attention": (ATTENTION_ONLY, 3), "scan": (SCAN_ONLY, 4),
+# a latent wider than any MFMA attention kernel's head: the plain attention kernel runs it
+WIDE_LATENT = model_config([latent(2, 8, 8, 16, 136, 0.3)], width=32, vocab=53)
+CONFIGS = {"wide": (WIDE_LATENT, 8), "mixed": (MIXED, 1), "odd": (ODD, 2), "attention": (ATTENTION_ONLY, 3), "scan": (SCAN_ONLY, 4),
            "heads": (HEADS_ONLY, 5), "ff": (FEED_FORWARD, 6), "ones": (ONES, 7)}
 
 _weights, _models = {}, {}
