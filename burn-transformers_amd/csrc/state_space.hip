@@ -224,13 +224,35 @@ struct SelectiveScanCall {
   int64_t state_stride;
   const int* seq_off;
   const int* slots;
+  // span > 0: long sequences are cut into spans of that many tokens which are scanned side by side
+  // (see "Spans" below); max_count is the most tokens a sequence of the step brings, carry the room
+  // for the spans' states: (tokens / span + 2 n_seqs + 1) blocks of channels * state + channels floats
+  int span;
+  int max_count;
+  float* carry;
 };
+
+// Spans.  A recurrence S_t = a_t S_(t-1) + u_t is linear in S, so a long sequence need not be walked
+// by one wave: cut into spans of `span` tokens, (1) every span is scanned from a zero state, side by
+// side, and leaves its end state E_k and the sum of its step sizes (its decays multiply up to
+// P_k = exp(A * that sum)); (2) a short kernel carries the state across the spans in order,
+// C_k = P_k C_(k-1) + E_k, from the slot's state; (3) every span is scanned again, side by side, from
+// the state C_(k-1) it really starts with, and writes the outputs.  The carrying kernel also keeps the
+// state the sequence came with (as "span -1": the third pass reads only the carry, never the slot, which
+// by then holds the state after the sequence's last token, written by the carrying kernel).  Twice the
+// arithmetic, on (sequence length / span) times the waves.  Span k of sequence s keeps its block at
+// index seq_off[s] / span + 2 s + 1 + k: ranges of different sequences do not meet.
+__device__ __forceinline__ int64_t span_block(const int* seq_off, int seq, int span, int part) {
+  return (int64_t)(seq_off[seq] / span + 2 * seq + 1 + part);
+}
 
 // LDS holds a run of `chunk` tokens' inputs (B and C rows padded to 8 R with zeros, and the wave's eight
 // channels' dt, x and z), brought in with loads that are all in flight together: one round trip to
 // memory per run of tokens instead of one per token, which is what bounds a recurrence.
+// phase 0: whole sequences, from and to the slot's state.  1: spans from zero, leaving E_k and the sum
+// of dt.  3: spans from the carried states, writing outputs.
 template <typename T, int R>
-__global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c, int chunk) {
+__global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c, int chunk, int phase) {
   extern __shared__ float lds[];
   constexpr int NP = 8 * R;
   float2* BC = reinterpret_cast<float2*>(lds);   // [chunk][NP] pairs (B, C): one 8-byte read for both
@@ -241,15 +263,26 @@ __global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c,
   const int ch = blockIdx.x * 8 + cl, seq = blockIdx.y;
   const bool live = ch < c.channels;
   const int chs = live ? ch : c.channels - 1;        // idle lanes read a valid channel and write nothing
-  const int first = c.seq_off[seq], last = c.seq_off[seq + 1];
+  int first = c.seq_off[seq], last = c.seq_off[seq + 1];
+  const int seq_last = last, part = blockIdx.z;
+  const int64_t per_span = (int64_t)c.channels * c.state + c.channels;
+  float* mine = nullptr;                             // this span's block of the carry
+  if (phase) {
+    first += part * c.span;
+    if (first >= seq_last) return;
+    last = min(first + c.span, seq_last);
+    mine = c.carry + span_block(c.seq_off, seq, c.span, part) * per_span;
+  }
   float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + (int64_t)chs * c.state;
+  const float* start = phase == 3 ? mine - per_span + (int64_t)chs * c.state : held;
   float A[R], S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int n = sub + 8 * r;
     A[r] = n < c.state ? -expf(c.A_log[(int64_t)chs * c.state + n]) : 0.f;
-    S[r] = n < c.state ? held[n] : 0.f;
+    S[r] = (n < c.state && phase != 1) ? start[n] : 0.f;
   }
+  float dt_sum = 0.f;
   const float Dc = c.D[chs];
   T* out = static_cast<T*>(c.out);
   for (int t0 = first; t0 < last; t0 += chunk) {
@@ -301,6 +334,8 @@ __global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c,
         S[r] = expf(dt * A[r]) * S[r] + dx * bc.x;
         acc = fmaf(S[r], bc.y, acc);
       }
+      dt_sum += dt;
+      if (phase == 1) return;                        // only the state is wanted
       acc = sum_of_8_lanes(acc);
       if (live && sub == 0)
         out[(int64_t)(t0 + i) * c.ld_out + ch] = from_float<T>((acc + Dc * xv) * silu_f(zs[i * 8 + cl]));
@@ -315,7 +350,18 @@ __global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c,
     }
     for (; i < count; ++i) token(i);
   }
-  if (live) {
+  if (phase == 1) {
+    if (live) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int n = sub + 8 * r;
+        if (n < c.state) mine[(int64_t)ch * c.state + n] = S[r];
+      }
+      if (sub == 0) mine[(int64_t)c.channels * c.state + ch] = dt_sum;
+    }
+    return;
+  }
+  if (live && phase == 0) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int n = sub + 8 * r;
@@ -335,12 +381,48 @@ static int scan_chunk(int floats_per_token, int tokens) {
   return chunk < tokens ? chunk : tokens;
 }
 
+// C_k = exp(A * sum of dt of span k) * C_(k-1) + E_k along every sequence, in place; C_(-1), the state the
+// sequence came with, is kept in front of its spans, and the last C goes into the slot.
+__global__ void __launch_bounds__(256) selective_carry_kernel(SelectiveScanCall c) {
+  const int seq = blockIdx.y;
+  const int64_t index = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, size = (int64_t)c.channels * c.state;
+  if (index >= size) return;
+  const int count = c.seq_off[seq + 1] - c.seq_off[seq];
+  const int spans = (count + c.span - 1) / c.span;
+  const int64_t per_span = size + c.channels;
+  float* block = c.carry + span_block(c.seq_off, seq, c.span, 0) * per_span;
+  float* slot = c.S + (int64_t)c.slots[seq] * c.state_stride;
+  float state = slot[index];
+  (block - per_span)[index] = state;
+  const float A = -expf(c.A_log[index]);
+  const int ch = (int)(index / c.state);
+  for (int k = 0; k < spans; ++k, block += per_span) {
+    state = expf(A * block[size + ch]) * state + block[index];
+    block[index] = state;
+  }
+  slot[index] = state;
+}
+
+// Sequences of at least this many spans are cut (fewer gain nothing over walking them).
+#define MIN_SPANS 3
+
 template <typename T, int R>
 static void launch_selective_scan_r(hipStream_t stream, const SelectiveScanCall& c) {
   const int per_token = 2 * 8 * R + 24;
+  dim3 block(64);
+  if (c.span > 0 && c.carry && c.max_count >= MIN_SPANS * c.span) {
+    const int chunk = scan_chunk(per_token, c.span);
+    const int spans = (c.max_count + c.span - 1) / c.span;
+    dim3 grid((c.channels + 7) / 8, c.n_seqs, spans);
+    const size_t lds = (size_t)chunk * per_token * sizeof(float);
+    hipLaunchKernelGGL((selective_scan_kernel<T, R>), grid, block, lds, stream, c, chunk, 1);
+    hipLaunchKernelGGL(selective_carry_kernel, dim3((c.channels * c.state + 255) / 256, c.n_seqs), dim3(256), 0, stream, c);
+    hipLaunchKernelGGL((selective_scan_kernel<T, R>), grid, block, lds, stream, c, chunk, 3);
+    return;
+  }
   const int chunk = scan_chunk(per_token, c.tokens);
-  dim3 grid((c.channels + 7) / 8, c.n_seqs), block(64);
-  hipLaunchKernelGGL((selective_scan_kernel<T, R>), grid, block, (size_t)chunk * per_token * sizeof(float), stream, c, chunk);
+  dim3 grid((c.channels + 7) / 8, c.n_seqs);
+  hipLaunchKernelGGL((selective_scan_kernel<T, R>), grid, block, (size_t)chunk * per_token * sizeof(float), stream, c, chunk, 0);
 }
 
 template <typename T>
@@ -391,13 +473,18 @@ struct HeadScanCall {
   int64_t state_stride;
   const int* seq_off;
   const int* slots;
+  // spans, as in SelectiveScanCall: a block of the carry holds a state (in the slot's layout) and, behind
+  // it, one number a head: the sum over the span of the logarithms of its decays
+  int span;
+  int max_count;
+  float* carry;
 };
 
 // The state of a slot is laid out for this kernel's lanes: [heads][tiles of 4 channels][state][4], so
 // that a wave's load of one register's worth of state (16 state elements by 4 channels) is 256
 // contiguous bytes.  Nobody else reads it; a new sequence's state is all zeros in any layout.
 template <int R>
-__global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk) {
+__global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk, int phase, int spans) {
   extern __shared__ float lds[];
   constexpr int NP = 16 * R;
   float2* BC = reinterpret_cast<float2*>(lds);   // [chunk][NP] pairs (B, C): one 8-byte read for both
@@ -405,18 +492,31 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
   float* steps = xs + (size_t)chunk * 4;   // [chunk] dt after bias and softplus
   float* decays = steps + chunk;           // [chunk]
   const int lane = threadIdx.x, sub = lane & 15, pl = lane >> 4;
-  const int tile = blockIdx.x, tiles = gridDim.x, head = blockIdx.y, seq = blockIdx.z;
+  const int tile = blockIdx.x, tiles = gridDim.x, head = blockIdx.y;
+  const int seq = blockIdx.z / spans, part = blockIdx.z % spans;
   const int p = tile * 4 + pl;
   const bool live = p < c.vdim;
   const int group = head / (c.heads / c.groups);
-  const int first = c.seq_off[seq], last = c.seq_off[seq + 1];
-  float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + ((int64_t)head * tiles + tile) * c.state * 4 + pl;
+  int first = c.seq_off[seq], last = c.seq_off[seq + 1];
+  const int seq_last = last;
+  const int64_t state_size = (int64_t)c.heads * tiles * c.state * 4, per_span = state_size + c.heads;
+  const int64_t in_state = ((int64_t)head * tiles + tile) * c.state * 4 + pl;
+  float* mine = nullptr;                             // this span's block of the carry
+  if (phase) {
+    first += part * c.span;
+    if (first >= seq_last) return;
+    last = min(first + c.span, seq_last);
+    mine = c.carry + span_block(c.seq_off, seq, c.span, part) * per_span;
+  }
+  float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + in_state;
+  const float* start = phase == 3 ? mine - per_span + in_state : held;
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int n = sub + 16 * r;
-    S[r] = n < c.state ? held[(int64_t)n * 4] : 0.f;
+    S[r] = (n < c.state && phase != 1) ? start[(int64_t)n * 4] : 0.f;
   }
+  float log_decay = 0.f;
   const float rate = -expf(c.A_log[head]), bias = c.dt_bias[head], Dh = c.D[head];
   const float* Bg = c.B + group * c.state;
   const float* Cg = c.C + group * c.state;
@@ -458,6 +558,8 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
         S[r] = decay * S[r] + dx * bc.x;
         acc = fmaf(S[r], bc.y, acc);
       }
+      log_decay += rate * steps[i];
+      if (phase == 1) return;                        // only the state is wanted
       acc = sum_of_16_lanes(acc);
       if (live && sub == 0) ycol[(int64_t)(t0 + i) * c.ld_y] = acc + Dh * xv;
     };
@@ -469,19 +571,64 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
     }
     for (; i < count; ++i) token(i);
   }
+  if (phase == 1) {
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int n = sub + 16 * r;
-    if (n < c.state) held[(int64_t)n * 4] = S[r];
+    for (int r = 0; r < R; ++r) {
+      const int n = sub + 16 * r;
+      if (n < c.state) mine[in_state + (int64_t)n * 4] = S[r];
+    }
+    if (tile == 0 && lane == 0) mine[state_size + head] = log_decay;
+    return;
   }
+  if (phase == 0) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = sub + 16 * r;
+      if (n < c.state) held[(int64_t)n * 4] = S[r];
+    }
+  }
+}
+
+// C_k = exp(sum of the span's log decays) * C_(k-1) + E_k along every sequence, in place (see selective_carry_kernel).
+__global__ void __launch_bounds__(256) head_carry_kernel(HeadScanCall c, int tiles) {
+  const int seq = blockIdx.y;
+  const int64_t per_head = (int64_t)tiles * c.state * 4, size = per_head * c.heads;
+  const int64_t index = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (index >= size) return;
+  const int count = c.seq_off[seq + 1] - c.seq_off[seq];
+  const int spans = (count + c.span - 1) / c.span;
+  const int64_t per_span = size + c.heads;
+  float* block = c.carry + span_block(c.seq_off, seq, c.span, 0) * per_span;
+  float* slot = c.S + (int64_t)c.slots[seq] * c.state_stride;
+  float state = slot[index];
+  (block - per_span)[index] = state;
+  const int head = (int)(index / per_head);
+  for (int k = 0; k < spans; ++k, block += per_span) {
+    state = expf(block[size + head]) * state + block[index];
+    block[index] = state;
+  }
+  slot[index] = state;
 }
 
 template <int R>
 static void launch_head_scan_r(hipStream_t stream, const HeadScanCall& c) {
   const int per_token = 2 * 16 * R + 6;
+  const int tiles = (c.vdim + 3) / 4;
+  dim3 block(64);
+  if (c.span > 0 && c.carry && c.max_count >= MIN_SPANS * c.span) {
+    const int chunk = scan_chunk(per_token, c.span);
+    const int spans = (c.max_count + c.span - 1) / c.span;
+    dim3 grid(tiles, c.heads, c.n_seqs * spans);
+    const size_t lds = (size_t)chunk * per_token * sizeof(float);
+    hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, lds, stream, c, chunk, 1, spans);
+    const int64_t size = (int64_t)c.heads * tiles * c.state * 4;
+    hipLaunchKernelGGL(head_carry_kernel, dim3((unsigned)((size + 255) / 256), c.n_seqs), dim3(256), 0, stream, c, tiles);
+    hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, lds, stream, c, chunk, 3, spans);
+    return;
+  }
   const int chunk = scan_chunk(per_token, c.tokens);
-  dim3 grid((c.vdim + 3) / 4, c.heads, c.n_seqs), block(64);
-  hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, (size_t)chunk * per_token * sizeof(float), stream, c, chunk);
+  dim3 grid(tiles, c.heads, c.n_seqs);
+  hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, (size_t)chunk * per_token * sizeof(float), stream, c, chunk, 0, 1);
 }
 
 BT_EXPORT int bt_head_scan_call(void* stream, const HeadScanCall* c) {

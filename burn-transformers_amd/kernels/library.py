@@ -131,16 +131,17 @@ class SelectiveScanCall(ctypes.Structure):
                 ("out_cols", _c_int), ("x", _c_ptr), ("ld_x", _c_i64), ("z", _c_ptr), ("ld_z", _c_i64), ("dt", _c_ptr),
                 ("ld_dt", _c_i64), ("B", _c_ptr), ("C", _c_ptr), ("ld_bc", _c_i64), ("A_log", _c_ptr), ("D", _c_ptr),
                 ("out", _c_ptr), ("ld_out", _c_i64), ("S", _c_ptr), ("state_stride", _c_i64), ("seq_off", _c_ptr),
-                ("slots", _c_ptr)]
-    _step_fields_ = {"tokens": "tokens"}
+                ("slots", _c_ptr), ("span", _c_int), ("max_count", _c_int), ("carry", _c_ptr)]
+    _step_fields_ = {"tokens": "tokens", "max_count": "max_count"}
 
 
 class HeadScanCall(ctypes.Structure):
     _fields_ = [("tokens", _c_int), ("n_seqs", _c_int), ("heads", _c_int), ("vdim", _c_int), ("state", _c_int),
                 ("groups", _c_int), ("x", _c_ptr), ("B", _c_ptr), ("C", _c_ptr), ("ld", _c_i64), ("dt_raw", _c_ptr),
                 ("ld_dt", _c_i64), ("dt_bias", _c_ptr), ("A_log", _c_ptr), ("D", _c_ptr), ("y", _c_ptr),
-                ("ld_y", _c_i64), ("S", _c_ptr), ("state_stride", _c_i64), ("seq_off", _c_ptr), ("slots", _c_ptr)]
-    _step_fields_ = {"tokens": "tokens"}
+                ("ld_y", _c_i64), ("S", _c_ptr), ("state_stride", _c_i64), ("seq_off", _c_ptr), ("slots", _c_ptr),
+                ("span", _c_int), ("max_count", _c_int), ("carry", _c_ptr)]
+    _step_fields_ = {"tokens": "tokens", "max_count": "max_count"}
 
 
 class GatedNormCall(ctypes.Structure):
@@ -1053,9 +1054,24 @@ def dt_project(low, weight, bias, out):
                           bias=bias.data_ptr(), out=out.data_ptr(), ld_out=out.stride(0)))
 
 
-def selective_scan(x, z, dt, B, C, A_log, D, out, state, step):
+SCAN_SPAN = 64        # tokens of a span of a long sequence (sequences of three spans or more are cut); 0: never cut
+
+
+def scan_carry(step, state_floats, extra_floats):
+    """Room for the states of the spans a step's long sequences are cut into (csrc/state_space.hip,
+    "Spans"): one block a span and one more a sequence; at most tokens / span + sequences spans exist
+    in a step of any shape of its class.  None for steps that are too short to be cut."""
+    if not SCAN_SPAN or step.token_capacity < 3 * SCAN_SPAN or step.max_count <= 1:
+        return None
+    blocks = step.token_capacity // SCAN_SPAN + 2 * step.n_seqs + 2
+    return step.buffer("scan.carry", blocks, state_floats + extra_floats, "float32")
+
+
+def selective_scan(x, z, dt, B, C, A_log, D, out, state, step, carry=None):
     """The selective scan with one state row per channel (see csrc/state_space.hip), gated by
-    silu(z); ``state`` [slots, >= channels * state elements] float32 is read and left updated."""
+    silu(z); ``state`` [slots, >= channels * state elements] float32 is read and left updated.
+    ``carry``: room from ``scan_carry`` (channels * elements state floats, channels extra); with it
+    long sequences are scanned in spans side by side."""
     channels, elements = A_log.shape
     _launch(_module("state_space"), "bt_selective_scan_call",
             SelectiveScanCall(out_dtype=DTYPE_CODES[out.dtype], tokens=x.shape[0], n_seqs=step.n_seqs, channels=channels,
@@ -1063,10 +1079,11 @@ def selective_scan(x, z, dt, B, C, A_log, D, out, state, step):
                               ld_z=z.stride(0), dt=dt.data_ptr(), ld_dt=dt.stride(0), B=B.data_ptr(), C=C.data_ptr(),
                               ld_bc=B.stride(0), A_log=A_log.data_ptr(), D=D.data_ptr(), out=out.data_ptr(),
                               ld_out=out.stride(0), S=state.data_ptr(), state_stride=state.stride(0),
-                              seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr()))
+                              seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr(),
+                              span=SCAN_SPAN if carry is not None else 0, max_count=step.max_count, carry=_ptr(carry)))
 
 
-def head_scan(x, B, C, dt_raw, dt_bias, A_log, D, y, state, step, heads, vdim, elements, groups):
+def head_scan(x, B, C, dt_raw, dt_bias, A_log, D, y, state, step, heads, vdim, elements, groups, carry=None):
     """The scan with one decay per head (see csrc/state_space.hip); x, B and C are column ranges of
     the same float32 rows; ``state`` [slots, >= heads * elements * vdim rounded up to 4] float32, in a
     layout of the kernel's own."""
@@ -1077,7 +1094,8 @@ def head_scan(x, B, C, dt_raw, dt_bias, A_log, D, y, state, step, heads, vdim, e
                          x=x.data_ptr(), B=B.data_ptr(), C=C.data_ptr(), ld=x.stride(0), dt_raw=dt_raw.data_ptr(),
                          ld_dt=dt_raw.stride(0), dt_bias=dt_bias.data_ptr(), A_log=A_log.data_ptr(), D=D.data_ptr(),
                          y=y.data_ptr(), ld_y=y.stride(0), S=state.data_ptr(), state_stride=state.stride(0),
-                         seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr()))
+                         seq_off=step.seq_off.data_ptr(), slots=step.slots.data_ptr(),
+                         span=SCAN_SPAN if carry is not None else 0, max_count=step.max_count, carry=_ptr(carry)))
 
 
 def gated_norm(y, z, weight, parts, eps, out):

@@ -93,7 +93,8 @@ class SelectiveScan(_Recurrent):
         K.dt_project(low[:, :self.dt_rank], self.dt_weight, self.dt_bias, dt)
         gated = step.buffer("scan.gated", tokens, self.inner_cols, step.dtype)
         K.selective_scan(x, xz[:, inner:], dt, low[:, self.dt_rank:self.dt_rank + self.state],
-                         low[:, self.dt_rank + self.state:], self.A_log, self.D, gated, scan_state, step)
+                         low[:, self.dt_rank + self.state:], self.A_log, self.D, gated, scan_state, step,
+                         carry=K.scan_carry(step, self.scan_state, inner))
         stream.add_product(step, gated, self.out_weight, packed=self.out_packed)
 
 
@@ -139,7 +140,8 @@ class HeadScan(_Recurrent):
         K.causal_conv(fused[:, inner:inner + self.channels], self.conv_weight, self.conv_bias, xbc, conv_state, step)
         y = step.buffer("scan.y", tokens, inner, "float32")
         K.head_scan(xbc[:, :inner], xbc[:, inner:inner + bc], xbc[:, inner + bc:], fused[:, inner + self.channels:],
-                    self.dt_bias, self.A_log, self.D, y, scan_state, step, self.heads, self.vdim, self.state, self.groups)
+                    self.dt_bias, self.A_log, self.D, y, scan_state, step, self.heads, self.vdim, self.state, self.groups,
+                    carry=K.scan_carry(step, self.scan_state, self.heads))
         gated = step.buffer("scan.gated", tokens, self.inner_cols, step.dtype)
         K.gated_norm(y, fused[:, :inner], self.norm_weight, self.norm_groups, self.eps, gated)
         stream.add_product(step, gated, self.out_weight, packed=self.out_packed)

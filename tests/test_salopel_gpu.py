@@ -297,3 +297,45 @@ def test_command_line(capsys, tmp_path):
     weights = weights_for("mixed")
     assert [line["token_ids"] for line in lines] == [plain.greedy(p, weights, config, 5) for p in prompts]
     assert main([str(tmp_path / "made"), text, "4", "--temperature", "0.7", "--seed", "5", "--prefill-chunk-size", "4"]) == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,lengths", [("scan", [200, 449]), ("heads", [193, 450]), ("mixed", [5, 257, 70, 400]),
+                                          ("odd", [260, 1, 199])])
+def test_long_prompts_whose_scans_run_in_spans(name, dtype, lengths):
+    """Prompts long enough for the recurrent layers to cut them into spans that are scanned side by
+    side, beside short ones in the same step; then a portion and single tokens from the state the
+    spans left; then the same sequences again in the slots given back."""
+    engine = engine_for(name, dtype, max_tokens=4096)
+    for round_ in range(2):
+        prompts = prompts_for(name, lengths, seed=70 + round_)
+        extra = prompts_for(name, [200 if n > 250 else 3 for n in lengths], seed=80 + round_)
+        slots = [engine.open() for _ in prompts]
+        logits = engine.step(list(zip(slots, prompts)), want=[list(range(len(p))) for p in prompts]).clone()
+        more = engine.step(list(zip(slots, extra)), want=[list(range(len(p))) for p in extra]).clone()
+        last = engine.step([(slot, [7]) for slot in slots]).clone()
+        at = at_more = 0
+        for i, (p, e) in enumerate(zip(prompts, extra)):
+            want = plain_logits(name, p + e + [7])
+            got = torch.cat([logits[at:at + len(p)], more[at_more:at_more + len(e)], last[i:i + 1]])
+            check(got, want, dtype, f"{name} request {i} of {len(p)} + {len(e)} + 1 tokens")
+            at, at_more = at + len(p), at_more + len(e)
+        for slot in slots:
+            engine.close(slot)
+    engine.cache.ledger.check()
+
+
+def test_spans_and_one_walk_agree():
+    """The same long prompt with its scans cut into spans and walked in one piece: rounding apart."""
+    from burn_transformers_amd.kernels import library as K
+    ids = prompts_for("mixed", [500], seed=90)[0]
+    results = []
+    for span in (K.SCAN_SPAN, 0):
+        held, K.SCAN_SPAN = K.SCAN_SPAN, span
+        try:
+            engine = engine_for("mixed", "float32", graphs=False, programs=False)
+            results.append(whole(engine, ids).cpu().double())
+        finally:
+            K.SCAN_SPAN = held
+    assert not torch.equal(results[0], results[1])            # two different orders of the sums did run
+    assert float((results[0] - results[1]).abs().max()) < 2e-5 + 2e-5 * float(results[1].abs().max())
