@@ -406,18 +406,47 @@ __global__ void __launch_bounds__(256) selective_carry_kernel(SelectiveScanCall 
 // Sequences of at least this many spans are cut (fewer gain nothing over walking them).
 #define MIN_SPANS 3
 
+static int simd_count() {
+  static int count = 0;
+  if (count == 0) {
+    int device = 0, units = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || units <= 0)
+      units = 256;
+    count = 4 * units;
+  }
+  return count;
+}
+
+// Into spans of how many tokens a step's long sequences are cut, 0 for not at all.  Spans double the
+// arithmetic, so they pay only while whole sequences leave the chip idle: `waves` (the waves that
+// walk whole sequences) must be at most half the SIMDs (measured at 1,024 waves on 1,024 SIMDs: the
+// head scan of 2 x 1,024 tokens took 666 us in 16 spans against 462 us whole; the selective scan,
+// 512 waves, 176 against 334 us), and there are as many spans as bring four waves to a SIMD, none
+// shorter than the call's `span`, which its room for the spans' states was sized for.
+static int span_tokens(int span, int max_count, const float* carry, int64_t waves) {
+  if (span <= 0 || !carry || waves * 2 > simd_count()) return 0;
+  const int64_t wanted = 4 * (int64_t)simd_count() / waves;
+  int tokens = (int)((max_count + wanted - 1) / wanted);
+  if (tokens < span) tokens = span;
+  return max_count >= MIN_SPANS * tokens ? tokens : 0;
+}
+
 template <typename T, int R>
 static void launch_selective_scan_r(hipStream_t stream, const SelectiveScanCall& c) {
   const int per_token = 2 * 8 * R + 24;
   dim3 block(64);
-  if (c.span > 0 && c.carry && c.max_count >= MIN_SPANS * c.span) {
-    const int chunk = scan_chunk(per_token, c.span);
-    const int spans = (c.max_count + c.span - 1) / c.span;
+  const int span = span_tokens(c.span, c.max_count, c.carry, (int64_t)((c.channels + 7) / 8) * c.n_seqs);
+  if (span > 0) {
+    SelectiveScanCall cut = c;
+    cut.span = span;
+    const int chunk = scan_chunk(per_token, span);
+    const int spans = (c.max_count + span - 1) / span;
     dim3 grid((c.channels + 7) / 8, c.n_seqs, spans);
     const size_t lds = (size_t)chunk * per_token * sizeof(float);
-    hipLaunchKernelGGL((selective_scan_kernel<T, R>), grid, block, lds, stream, c, chunk, 1);
-    hipLaunchKernelGGL(selective_carry_kernel, dim3((c.channels * c.state + 255) / 256, c.n_seqs), dim3(256), 0, stream, c);
-    hipLaunchKernelGGL((selective_scan_kernel<T, R>), grid, block, lds, stream, c, chunk, 3);
+    hipLaunchKernelGGL((selective_scan_kernel<T, R>), grid, block, lds, stream, cut, chunk, 1);
+    hipLaunchKernelGGL(selective_carry_kernel, dim3((c.channels * c.state + 255) / 256, c.n_seqs), dim3(256), 0, stream, cut);
+    hipLaunchKernelGGL((selective_scan_kernel<T, R>), grid, block, lds, stream, cut, chunk, 3);
     return;
   }
   const int chunk = scan_chunk(per_token, c.tokens);
@@ -615,15 +644,18 @@ static void launch_head_scan_r(hipStream_t stream, const HeadScanCall& c) {
   const int per_token = 2 * 16 * R + 6;
   const int tiles = (c.vdim + 3) / 4;
   dim3 block(64);
-  if (c.span > 0 && c.carry && c.max_count >= MIN_SPANS * c.span) {
-    const int chunk = scan_chunk(per_token, c.span);
-    const int spans = (c.max_count + c.span - 1) / c.span;
+  const int span = span_tokens(c.span, c.max_count, c.carry, (int64_t)tiles * c.heads * c.n_seqs);
+  if (span > 0) {
+    HeadScanCall cut = c;
+    cut.span = span;
+    const int chunk = scan_chunk(per_token, span);
+    const int spans = (c.max_count + span - 1) / span;
     dim3 grid(tiles, c.heads, c.n_seqs * spans);
     const size_t lds = (size_t)chunk * per_token * sizeof(float);
-    hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, lds, stream, c, chunk, 1, spans);
+    hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, lds, stream, cut, chunk, 1, spans);
     const int64_t size = (int64_t)c.heads * tiles * c.state * 4;
-    hipLaunchKernelGGL(head_carry_kernel, dim3((unsigned)((size + 255) / 256), c.n_seqs), dim3(256), 0, stream, c, tiles);
-    hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, lds, stream, c, chunk, 3, spans);
+    hipLaunchKernelGGL(head_carry_kernel, dim3((unsigned)((size + 255) / 256), c.n_seqs), dim3(256), 0, stream, cut, tiles);
+    hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, lds, stream, cut, chunk, 3, spans);
     return;
   }
   const int chunk = scan_chunk(per_token, c.tokens);
