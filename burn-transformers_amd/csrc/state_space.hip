@@ -512,14 +512,12 @@ struct HeadScanCall {
 // The state of a slot is laid out for this kernel's lanes: [heads][tiles of 4 channels][state][4], so
 // that a wave's load of one register's worth of state (16 state elements by 4 channels) is 256
 // contiguous bytes.  Nobody else reads it; a new sequence's state is all zeros in any layout.
-template <int R>
-__global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk, int phase, int spans) {
+template <int R, int PHASE>
+__global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk, int spans) {
   extern __shared__ float lds[];
   constexpr int NP = 16 * R;
-  float2* BC = reinterpret_cast<float2*>(lds);   // [chunk][NP] pairs (B, C): one 8-byte read for both
-  float* xs = lds + (size_t)chunk * NP * 2;      // [chunk][4]
-  float* steps = xs + (size_t)chunk * 4;   // [chunk] dt after bias and softplus
-  float* decays = steps + chunk;           // [chunk]
+  float2* BC = reinterpret_cast<float2*>(lds);                              // [chunk][NP] pairs (B, C): one 8-byte read for both
+  float4* tok = reinterpret_cast<float4*>(lds + (size_t)chunk * NP * 2);    // [chunk][4]: a token and channel's dt * x, D * x, decay, log decay
   const int lane = threadIdx.x, sub = lane & 15, pl = lane >> 4;
   const int tile = blockIdx.x, tiles = gridDim.x, head = blockIdx.y;
   const int seq = blockIdx.z / spans, part = blockIdx.z % spans;
@@ -531,19 +529,19 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
   const int64_t state_size = (int64_t)c.heads * tiles * c.state * 4, per_span = state_size + c.heads;
   const int64_t in_state = ((int64_t)head * tiles + tile) * c.state * 4 + pl;
   float* mine = nullptr;                             // this span's block of the carry
-  if (phase) {
+  if (PHASE) {
     first += part * c.span;
     if (first >= seq_last) return;
     last = min(first + c.span, seq_last);
     mine = c.carry + span_block(c.seq_off, seq, c.span, part) * per_span;
   }
   float* held = c.S + (int64_t)c.slots[seq] * c.state_stride + in_state;
-  const float* start = phase == 3 ? mine - per_span + in_state : held;
+  const float* start = PHASE == 3 ? mine - per_span + in_state : held;
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int n = sub + 16 * r;
-    S[r] = (n < c.state && phase != 1) ? start[(int64_t)n * 4] : 0.f;
+    S[r] = (n < c.state && PHASE != 1) ? start[(int64_t)n * 4] : 0.f;
   }
   float log_decay = 0.f;
   const float rate = -expf(c.A_log[head]), bias = c.dt_bias[head], Dh = c.D[head];
@@ -569,38 +567,46 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
     }
     for (int e = lane; e < count * 4; e += 64) {
       const int i = e >> 2, q = tile * 4 + (e & 3);
-      xs[e] = q < c.vdim ? c.x[(int64_t)(t0 + i) * c.ld + head * c.vdim + q] : 0.f;
-    }
-    for (int e = lane; e < count; e += 64) {
-      const float step = softplus_f(c.dt_raw[(int64_t)(t0 + e) * c.ld_dt + head] + bias);
-      steps[e] = step;
-      decays[e] = expf(rate * step);
+      const float xv = q < c.vdim ? c.x[(int64_t)(t0 + i) * c.ld + head * c.vdim + q] : 0.f;
+      const float step = softplus_f(c.dt_raw[(int64_t)(t0 + i) * c.ld_dt + head] + bias);
+      tok[e] = make_float4(step * xv, Dh * xv, expf(rate * step), rate * step);
     }
     __syncthreads();
-    auto token = [&](int i) {
-      const float xv = xs[i * 4 + pl], decay = decays[i];
-      const float dx = steps[i] * xv;
+    // one token: the state moves on; the channel's output (in every lane of its sixteen) is returned
+    auto token = [&](int i) -> float {
+      const float4 in = tok[i * 4 + pl];
       float acc = 0.f;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const float2 bc = BC[i * NP + sub + 16 * r];
-        S[r] = decay * S[r] + dx * bc.x;
+        S[r] = fmaf(in.z, S[r], in.x * bc.x);
         acc = fmaf(S[r], bc.y, acc);
       }
-      log_decay += rate * steps[i];
-      if (phase == 1) return;                        // only the state is wanted
-      acc = sum_of_16_lanes(acc);
-      if (live && sub == 0) ycol[(int64_t)(t0 + i) * c.ld_y] = acc + Dh * xv;
+      if (PHASE == 1) {
+        log_decay += in.w;
+        return 0.f;                                  // only the state is wanted
+      }
+      return sum_of_16_lanes(acc) + in.y;
     };
-    // four tokens at a time, written out (see selective_scan_kernel)
+    // Sixteen tokens at a time, written out: their reads from LDS and sums are in flight together and
+    // only the state ties them (the lane sums keep the compiler from unrolling a loop whose length it
+    // does not know); lane j of a channel's sixteen keeps the j-th of them, and one store writes all.
     int i = 0;
-    for (; i + 4 <= count; i += 4) {
+    for (; i + 16 <= count; i += 16) {
+      float kept = 0.f;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) token(i + u);
+      for (int u = 0; u < 16; ++u) {
+        const float y = token(i + u);
+        kept = sub == u ? y : kept;
+      }
+      if (PHASE != 1 && live) ycol[(int64_t)(t0 + i + sub) * c.ld_y] = kept;
     }
-    for (; i < count; ++i) token(i);
+    for (; i < count; ++i) {
+      const float y = token(i);
+      if (PHASE != 1 && live && sub == 0) ycol[(int64_t)(t0 + i) * c.ld_y] = y;
+    }
   }
-  if (phase == 1) {
+  if (PHASE == 1) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int n = sub + 16 * r;
@@ -609,7 +615,7 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
     if (tile == 0 && lane == 0) mine[state_size + head] = log_decay;
     return;
   }
-  if (phase == 0) {
+  if (PHASE == 0) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int n = sub + 16 * r;
@@ -641,7 +647,7 @@ __global__ void __launch_bounds__(256) head_carry_kernel(HeadScanCall c, int til
 
 template <int R>
 static void launch_head_scan_r(hipStream_t stream, const HeadScanCall& c) {
-  const int per_token = 2 * 16 * R + 6;
+  const int per_token = 2 * 16 * R + 16;
   const int tiles = (c.vdim + 3) / 4;
   dim3 block(64);
   const int span = span_tokens(c.span, c.max_count, c.carry, (int64_t)tiles * c.heads * c.n_seqs);
@@ -652,15 +658,15 @@ static void launch_head_scan_r(hipStream_t stream, const HeadScanCall& c) {
     const int spans = (c.max_count + span - 1) / span;
     dim3 grid(tiles, c.heads, c.n_seqs * spans);
     const size_t lds = (size_t)chunk * per_token * sizeof(float);
-    hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, lds, stream, cut, chunk, 1, spans);
+    hipLaunchKernelGGL((head_scan_kernel<R, 1>), grid, block, lds, stream, cut, chunk, spans);
     const int64_t size = (int64_t)c.heads * tiles * c.state * 4;
     hipLaunchKernelGGL(head_carry_kernel, dim3((unsigned)((size + 255) / 256), c.n_seqs), dim3(256), 0, stream, cut, tiles);
-    hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, lds, stream, cut, chunk, 3, spans);
+    hipLaunchKernelGGL((head_scan_kernel<R, 3>), grid, block, lds, stream, cut, chunk, spans);
     return;
   }
   const int chunk = scan_chunk(per_token, c.tokens);
   dim3 grid(tiles, c.heads, c.n_seqs);
-  hipLaunchKernelGGL((head_scan_kernel<R>), grid, block, (size_t)chunk * per_token * sizeof(float), stream, c, chunk, 0, 1);
+  hipLaunchKernelGGL((head_scan_kernel<R, 0>), grid, block, (size_t)chunk * per_token * sizeof(float), stream, c, chunk, 1);
 }
 
 BT_EXPORT int bt_head_scan_call(void* stream, const HeadScanCall* c) {
