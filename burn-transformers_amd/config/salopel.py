@@ -6,7 +6,7 @@
     norm.eps       the epsilon of every norm of the model
     layers         a list; each entry has ``type`` (latent_attention | mamba1 | mamba2), ``mixer`` (the
                    mixer's sizes), ``mlp`` ({"kind": "dense", "ff": n} or null) and optionally
-                   ``weights_of``: the index of an earlier layer whose tensors it runs (with a cache
+                   ``weights_of``: the index of another layer whose tensors it runs (with a cache
                    or state of its own)
 
 Every size and constant of a model is one of these keys or a tensor's shape; nothing has a default.
@@ -119,19 +119,25 @@ class SalopelConfig:
                 if (sizes["heads"] * sizes["vdim"]) % sizes["norm_groups"] != 0:
                     raise ConfigError(FAMILY, f"{where}.mixer.norm_groups", "must divide heads * vdim")
             if layer.weights_of is not None:
-                owner = layer.weights_of
-                if not (0 <= owner < index):
-                    raise ConfigError(FAMILY, f"{where}.weights_of", "must name an earlier layer")
+                if not (0 <= layer.weights_of < len(self.layers)) or layer.weights_of == index:
+                    raise ConfigError(FAMILY, f"{where}.weights_of", "must name another layer of the model")
+                owner = self.owner(index)
+                if owner is None:
+                    raise ConfigError(FAMILY, f"{where}.weights_of", "leads round in a circle: no layer of it has tensors")
                 held = self.layers[owner]
-                if held.weights_of is not None:
-                    raise ConfigError(FAMILY, f"{where}.weights_of", f"layer {owner} has no tensors of its own")
                 if (held.type, held.mixer, held.ff) != (layer.type, layer.mixer, layer.ff):
                     raise ConfigError(FAMILY, f"{where}.weights_of", f"differs from layer {owner}, whose tensors it runs")
 
     def owner(self, index):
-        """The layer whose tensors layer ``index`` runs (itself unless it borrows)."""
-        owner = self.layers[index].weights_of
-        return index if owner is None else owner
+        """The layer whose tensors layer ``index`` runs: itself unless it borrows; a borrower may come
+        before or after its owner, and may name another borrower (None if that leads round in a circle)."""
+        seen = set()
+        while self.layers[index].weights_of is not None:
+            if index in seen:
+                return None
+            seen.add(index)
+            index = self.layers[index].weights_of
+        return index
 
     def to_dict(self):
         return {"architecture": "Salopel", "vocab": self.vocab, "width": self.width,

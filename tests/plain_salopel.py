@@ -147,8 +147,9 @@ def forward(ids, weights, config, dtype=torch.float64, layers_out=None):
     eps, mult = config["norm"]["eps"], config["residual_mult"]
     x = norm_around_zero(w["embed"][torch.as_tensor(ids, dtype=torch.long)], w["embed.norm"], eps)
     for index, entry in enumerate(config["layers"]):
-        owner = entry.get("weights_of")
-        layer = owner if owner is not None else index      # a borrower runs its owner's tensors
+        layer = index
+        while config["layers"][layer].get("weights_of") is not None:      # a borrower runs its owner's tensors
+            layer = config["layers"][layer]["weights_of"]
         x = x + mult * norm_around_zero(mixer(x, w, layer, entry, eps), w[f"l{layer}.norm1"], eps)
         if entry.get("mlp") is not None:
             x = x + mult * norm_around_zero(feed_forward(x, w, f"l{layer}.mlp.", eps), w[f"l{layer}.norm2"], eps)

@@ -61,7 +61,10 @@ HEADS_ONLY = model_config([mamba2(4, 16, 32, 2, 2, 4)], width=32, vocab=101, mul
 FEED_FORWARD = model_config([latent(1, 8, 8, 8, 16, 1.0, ff=40)], width=32, vocab=61, mult=2.0)
 # a latent wider than any MFMA attention kernel's head: the plain attention kernel runs it
 WIDE_LATENT = model_config([latent(2, 8, 8, 16, 136, 0.3)], width=32, vocab=53)
-CONFIGS = {"wide": (WIDE_LATENT, 8), "mixed": (MIXED, 1), "odd": (ODD, 2), "attention": (ATTENTION_ONLY, 3), "scan": (SCAN_ONLY, 4),
+# the first layer runs the third's tensors, the last one the second's: a borrower before and behind its owner
+LOOPED = model_config([latent(2, 16, 8, 24, 32, 0.3, ff=40, weights_of=2), mamba1(48, 8, 4, 3),
+                       latent(2, 16, 8, 24, 32, 0.3, ff=40), mamba1(48, 8, 4, 3, weights_of=1)], width=48, vocab=89)
+CONFIGS = {"looped": (LOOPED, 9), "wide": (WIDE_LATENT, 8), "mixed": (MIXED, 1), "odd": (ODD, 2), "attention": (ATTENTION_ONLY, 3), "scan": (SCAN_ONLY, 4),
            "heads": (HEADS_ONLY, 5), "ff": (FEED_FORWARD, 6), "ones": (ONES, 7)}
 
 _weights, _models = {}, {}

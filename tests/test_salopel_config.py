@@ -36,7 +36,8 @@ def test_configuration_round_trip(name):
     (lambda c: c["layers"][1]["mlp"].update(kind="experts"), "layers[1].mlp.kind"),
     (lambda c: c["layers"][3].update(weights_of=3), "layers[3].weights_of"),
     (lambda c: c["layers"][3].update(weights_of=1), "layers[3].weights_of"),
-    (lambda c: c["layers"][4].update(weights_of=3), "layers[4].weights_of"),
+    (lambda c: c["layers"][3].update(weights_of=9), "layers[3].weights_of"),
+    (lambda c: (c["layers"][0].update(weights_of=3), c["layers"][3].update(weights_of=0)), "layers[0].weights_of"),
 ])
 def test_each_bad_field_is_named(change, field):
     config = copy.deepcopy(MIXED)
@@ -118,3 +119,20 @@ def test_the_plain_convolution_and_polynorm():
     assert torch.allclose(got, z / (12.5 ** 0.5) + 0.25)
     got = plain.poly_norm(z, torch.tensor([0.0, 2.0, 0.0, 0.0], dtype=torch.float64), 0.0)
     assert torch.allclose(got, 2 * z * z / ((81 + 256) / 2) ** 0.5)
+
+
+def test_a_borrower_may_come_before_its_owner_or_name_another_borrower():
+    layers = [latent(2, 8, 8, 8, 16, 0.5, ff=24, weights_of=2), mamba1(24, 4, 2, 3), latent(2, 8, 8, 8, 16, 0.5, ff=24),
+              mamba1(24, 4, 2, 3, weights_of=1), mamba1(24, 4, 2, 3, weights_of=3)]
+    config_json = model_config(layers, width=16, vocab=29)
+    family = bt.resolve_family(config_json)
+    config = family.config_class.from_dict(config_json)
+    assert [config.owner(i) for i in range(5)] == [2, 1, 2, 1, 1]
+    plan = family.plan(config)
+    assert [(e.layer, e.cache) for e in plan.schedule] == [(1, 0), (0, 1), (1, 2), (0, 3), (0, 4)]
+    names = {spec.name for spec in family.contract(config).tensors}
+    assert any(n.startswith("l1.") for n in names) and any(n.startswith("l2.") for n in names)
+    assert not any(n.startswith(("l0.", "l3.", "l4.")) for n in names)
+    _, tensors = bt.random_tensors(config_json, 0)
+    logits = plain.forward([1, 2, 3, 4], tensors, config_json)
+    assert logits.shape == (4, 29) and torch.isfinite(logits).all()
