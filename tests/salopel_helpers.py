@@ -64,7 +64,11 @@ WIDE_LATENT = model_config([latent(2, 8, 8, 16, 136, 0.3)], width=32, vocab=53)
 # the first layer runs the third's tensors, the last one the second's: a borrower before and behind its owner
 LOOPED = model_config([latent(2, 16, 8, 24, 32, 0.3, ff=40, weights_of=2), mamba1(48, 8, 4, 3),
                        latent(2, 16, 8, 24, 32, 0.3, ff=40), mamba1(48, 8, 4, 3, weights_of=1)], width=48, vocab=89)
-CONFIGS = {"looped": (LOOPED, 9), "wide": (WIDE_LATENT, 8), "mixed": (MIXED, 1), "odd": (ODD, 2), "attention": (ATTENTION_ONLY, 3), "scan": (SCAN_ONLY, 4),
+# odd numbers everywhere a kernel counts in fours, eights or sixteens: head sizes 6 and 10, values of 5,
+# ranks 7 and 9, 3 heads in 3 groups, 30 and 18 inner channels, a feed-forward of 37
+RAGGED = model_config([mamba2(3, 6, 9, 3, 1, 2, ff=37), latent(3, 6, 5, 7, 9, 0.4), mamba1(30, 3, 5, 2),
+                       mamba2(1, 10, 17, 1, 2, 3), latent(5, 3, 7, 9, 11, 0.6, ff=19)], width=40, vocab=71, mult=0.9)
+CONFIGS = {"ragged": (RAGGED, 10), "looped": (LOOPED, 9), "wide": (WIDE_LATENT, 8), "mixed": (MIXED, 1), "odd": (ODD, 2), "attention": (ATTENTION_ONLY, 3), "scan": (SCAN_ONLY, 4),
            "heads": (HEADS_ONLY, 5), "ff": (FEED_FORWARD, 6), "ones": (ONES, 7)}
 
 _weights, _models = {}, {}

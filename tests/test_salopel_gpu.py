@@ -40,7 +40,7 @@ def whole(engine, ids):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name,lengths", [("attention", [1, 9, 70]), ("scan", [1, 2, 40]), ("heads", [1, 3, 40]),
                                           ("ff", [1, 17]), ("mixed", [1, 5, 66, 130]), ("odd", [1, 7, 90]),
-                                          ("wide", [1, 70]), ("looped", [1, 40])])
+                                          ("wide", [1, 70]), ("looped", [1, 40]), ("ragged", [1, 2, 75, 210])])
 def test_each_mechanism_and_each_request_whole(name, dtype, lengths):
     engine = engine_for(name, dtype)
     for ids in prompts_for(name, lengths):
@@ -50,7 +50,7 @@ def test_each_mechanism_and_each_request_whole(name, dtype, lengths):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name,length,tail", [("mixed", 80, 30), ("odd", 70, 12), ("scan", 9, 8), ("heads", 9, 8),
-                                              ("wide", 70, 8), ("looped", 30, 10)])
+                                              ("wide", 70, 8), ("looped", 30, 10), ("ragged", 70, 20)])
 def test_prompt_then_token_by_token(name, dtype, length, tail):
     """The last tokens one by one through cache and state give what the whole prompt gives."""
     engine = engine_for(name, dtype)
@@ -90,7 +90,7 @@ def test_from_the_first_token_one_by_one(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,chunk,length", [("mixed", 2, 21), ("mixed", 7, 100), ("mixed", 64, 150), ("odd", 3, 40),
+@pytest.mark.parametrize("name,chunk,length", [("ragged", 5, 33), ("ragged", 66, 200), ("mixed", 2, 21), ("mixed", 7, 100), ("mixed", 64, 150), ("odd", 3, 40),
                                                ("odd", 65, 140)])
 def test_prompts_in_portions(name, dtype, chunk, length):
     """Portions of a prompt, down to two tokens, each from what the one before left: the convolution's
