@@ -9,7 +9,52 @@
 //   * gate, then RMS norm in equal parts
 #include "host.h"
 
-#define FILL 16      // elements a lane brings into LDS at a time, with loads that are all in flight together
+
+// Brings rows t0 .. t0 + count - 1 of B and C (`state` columns each, row pitch `ld`, 32-bit offsets) into LDS
+// as pairs, [count][NP] with zeros behind `state`; NP is a power of two.  A pass of the wave covers
+// whole rows (64 / NP of them, or 1 / (NP / 64) of one), a lane keeps its column, and thirty-two passes'
+// loads are issued before the first is stored: a loop of single loads would wait for memory once per
+// element, and one that works its row and column out of a running index spends more instructions on
+// that than the recurrence spends on a token.
+template <int NP, int LOADS>
+__device__ __forceinline__ void fill_pairs_ahead(float2* BC, const float* B, const float* C, int ld, int t0, int count,
+                                                 int state, int lane) {
+  constexpr int ROWS = NP >= 64 ? 1 : 64 / NP;     // rows a pass covers
+  constexpr int COLS = NP >= 64 ? NP / 64 : 1;     // passes a row takes
+  constexpr int AHEAD = COLS >= LOADS ? 1 : LOADS / COLS;  // row passes whose loads are in flight together
+  const int lane_row = NP >= 64 ? 0 : lane / NP, lane_col = NP >= 64 ? lane : lane % NP;
+  for (int r0 = 0; r0 < count; r0 += ROWS * AHEAD) {
+    float2 got[AHEAD][COLS];
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int row = r0 + u * ROWS + lane_row;
+      const int at = (t0 + min(row, count - 1)) * ld;
+#pragma unroll
+      for (int k = 0; k < COLS; ++k) {
+        const int n = lane_col + 64 * k;
+        got[u][k] = (row < count && n < state) ? make_float2(B[at + n], C[at + n]) : make_float2(0.f, 0.f);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int row = r0 + u * ROWS + lane_row;
+#pragma unroll
+      for (int k = 0; k < COLS; ++k)
+        if (row < count) BC[row * NP + lane_col + 64 * k] = got[u][k];
+    }
+  }
+}
+
+// (a step of single tokens has one row to bring: the short form spares it the long one's idle passes)
+template <int NP>
+__device__ __forceinline__ void fill_pairs(float2* BC, const float* B, const float* C, int ld, int t0, int count,
+                                           int state, int lane) {
+  constexpr int ROWS = NP >= 64 ? 1 : 64 / NP;
+  if (count <= 2 * ROWS)
+    fill_pairs_ahead<NP, 2>(BC, B, C, ld, t0, count, state, lane);
+  else
+    fill_pairs_ahead<NP, 32>(BC, B, C, ld, t0, count, state, lane);
+}
 
 // Sums over groups of 8 or 16 neighbouring lanes with data-parallel moves between lanes of a row
 // (no trip through the LDS crossbar as a shuffle takes; a recurrence pays this once per token): first
@@ -288,19 +333,19 @@ __global__ void __launch_bounds__(64) selective_scan_kernel(SelectiveScanCall c,
   for (int t0 = first; t0 < last; t0 += chunk) {
     const int count = min(chunk, last - t0);
     __syncthreads();
-    // (several elements of a lane at a time, all loads issued before the first is stored: a loop of
-    // single loads would wait for memory once per element)
-    for (int e0 = lane; e0 < count * NP; e0 += 64 * FILL) {
-      float2 held_bc[FILL];
+    // (sixteen elements of a lane at a time, all loads issued before the first is stored; with the
+    // short rows of this scan, 8 to 32 pairs, the running index measured faster than `fill_pairs`)
+    for (int e0 = lane; e0 < count * NP; e0 += 64 * 16) {
+      float2 held_bc[16];
 #pragma unroll
-      for (int k = 0; k < FILL; ++k) {
+      for (int k = 0; k < 16; ++k) {
         const int e = e0 + 64 * k, i = e / NP, n = e % NP;
         held_bc[k] = (e < count * NP && n < c.state)
                          ? make_float2(c.B[(int64_t)(t0 + i) * c.ld_bc + n], c.C[(int64_t)(t0 + i) * c.ld_bc + n])
                          : make_float2(0.f, 0.f);
       }
 #pragma unroll
-      for (int k = 0; k < FILL; ++k)
+      for (int k = 0; k < 16; ++k)
         if (e0 + 64 * k < count * NP) BC[e0 + 64 * k] = held_bc[k];
     }
     {
@@ -551,20 +596,7 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
   for (int t0 = first; t0 < last; t0 += chunk) {
     const int count = min(chunk, last - t0);
     __syncthreads();
-    // (sixteen elements of a lane at a time, all loads issued before the first is stored: a loop of
-    // single loads would wait for memory once per element)
-    for (int e0 = lane; e0 < count * NP; e0 += 64 * FILL) {
-      float2 held_bc[FILL];
-#pragma unroll
-      for (int k = 0; k < FILL; ++k) {
-        const int e = e0 + 64 * k, i = e / NP, n = e % NP;
-        held_bc[k] = (e < count * NP && n < c.state)
-                         ? make_float2(Bg[(int64_t)(t0 + i) * c.ld + n], Cg[(int64_t)(t0 + i) * c.ld + n]) : make_float2(0.f, 0.f);
-      }
-#pragma unroll
-      for (int k = 0; k < FILL; ++k)
-        if (e0 + 64 * k < count * NP) BC[e0 + 64 * k] = held_bc[k];
-    }
+    fill_pairs<NP>(BC, Bg, Cg, (int)c.ld, t0, count, c.state, lane);
     for (int e = lane; e < count * 4; e += 64) {
       const int i = e >> 2, q = tile * 4 + (e & 3);
       const float xv = q < c.vdim ? c.x[(int64_t)(t0 + i) * c.ld + head * c.vdim + q] : 0.f;
@@ -678,6 +710,7 @@ BT_EXPORT int bt_head_scan_call(void* stream, const HeadScanCall* c) {
   if (c->ld_dt < c->heads || c->ld_y < (int64_t)c->heads * c->vdim ||
       c->state_stride < (int64_t)c->heads * c->state * ((c->vdim + 3) / 4 * 4))
     BT_REFUSE("head_scan: rows or state too short for %d heads of %d", c->heads, c->vdim);
+  if ((int64_t)c->tokens * c->ld >= (int64_t)1 << 31) BT_REFUSE("head_scan: the rows of B and C are addressed with 32 bits");
   hipStream_t s = (hipStream_t)stream;
   const int per = (c->state + 15) / 16;
   if (per <= 1) launch_head_scan_r<1>(s, *c);
