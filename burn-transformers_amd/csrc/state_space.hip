@@ -15,14 +15,14 @@
 // whole rows (64 / NP of them, or 1 / (NP / 64) of one), a lane keeps its column, and thirty-two passes'
 // loads are issued before the first is stored: a loop of single loads would wait for memory once per
 // element, and one that works its row and column out of a running index spends more instructions on
-// that than the recurrence spends on a token.
-template <int NP, int LOADS>
+// that than the recurrence spends on a token.  `lane` numbers the THREADS threads that share the work.
+template <int NP, int LOADS, int THREADS>
 __device__ __forceinline__ void fill_pairs_ahead(float2* BC, const float* B, const float* C, int ld, int t0, int count,
                                                  int state, int lane) {
-  constexpr int ROWS = NP >= 64 ? 1 : 64 / NP;     // rows a pass covers
-  constexpr int COLS = NP >= 64 ? NP / 64 : 1;     // passes a row takes
-  constexpr int AHEAD = COLS >= LOADS ? 1 : LOADS / COLS;  // row passes whose loads are in flight together
-  const int lane_row = NP >= 64 ? 0 : lane / NP, lane_col = NP >= 64 ? lane : lane % NP;
+  constexpr int ROWS = NP >= THREADS ? 1 : THREADS / NP;     // rows a pass covers
+  constexpr int COLS = NP >= THREADS ? NP / THREADS : 1;     // passes a row takes
+  constexpr int AHEAD = COLS >= LOADS ? 1 : LOADS / COLS;    // row passes whose loads are in flight together
+  const int lane_row = NP >= THREADS ? 0 : lane / NP, lane_col = NP >= THREADS ? lane : lane % NP;
   for (int r0 = 0; r0 < count; r0 += ROWS * AHEAD) {
     float2 got[AHEAD][COLS];
 #pragma unroll
@@ -31,7 +31,7 @@ __device__ __forceinline__ void fill_pairs_ahead(float2* BC, const float* B, con
       const int at = (t0 + min(row, count - 1)) * ld;
 #pragma unroll
       for (int k = 0; k < COLS; ++k) {
-        const int n = lane_col + 64 * k;
+        const int n = lane_col + THREADS * k;
         got[u][k] = (row < count && n < state) ? make_float2(B[at + n], C[at + n]) : make_float2(0.f, 0.f);
       }
     }
@@ -40,20 +40,20 @@ __device__ __forceinline__ void fill_pairs_ahead(float2* BC, const float* B, con
       const int row = r0 + u * ROWS + lane_row;
 #pragma unroll
       for (int k = 0; k < COLS; ++k)
-        if (row < count) BC[row * NP + lane_col + 64 * k] = got[u][k];
+        if (row < count) BC[row * NP + lane_col + THREADS * k] = got[u][k];
     }
   }
 }
 
 // (a step of single tokens has one row to bring: the short form spares it the long one's idle passes)
-template <int NP>
+template <int NP, int THREADS>
 __device__ __forceinline__ void fill_pairs(float2* BC, const float* B, const float* C, int ld, int t0, int count,
                                            int state, int lane) {
-  constexpr int ROWS = NP >= 64 ? 1 : 64 / NP;
+  constexpr int ROWS = NP >= THREADS ? 1 : THREADS / NP;
   if (count <= 2 * ROWS)
-    fill_pairs_ahead<NP, 2>(BC, B, C, ld, t0, count, state, lane);
+    fill_pairs_ahead<NP, 2, THREADS>(BC, B, C, ld, t0, count, state, lane);
   else
-    fill_pairs_ahead<NP, 32>(BC, B, C, ld, t0, count, state, lane);
+    fill_pairs_ahead<NP, 2048 / THREADS, THREADS>(BC, B, C, ld, t0, count, state, lane);
 }
 
 // Sums over groups of 8 or 16 neighbouring lanes with data-parallel moves between lanes of a row
@@ -464,14 +464,14 @@ static int simd_count() {
 }
 
 // Into spans of how many tokens a step's long sequences are cut, 0 for not at all.  Spans double the
-// arithmetic, so they pay only while whole sequences leave the chip idle: `waves` (the waves that
-// walk whole sequences) must be at most half the SIMDs (measured at 1,024 waves on 1,024 SIMDs: the
-// head scan of 2 x 1,024 tokens took 666 us in 16 spans against 462 us whole; the selective scan,
-// 512 waves, 176 against 334 us), and there are as many spans as bring four waves to a SIMD, none
-// shorter than the call's `span`, which its room for the spans' states was sized for.
-static int span_tokens(int span, int max_count, const float* carry, int64_t waves) {
-  if (span <= 0 || !carry || waves * 2 > simd_count()) return 0;
-  const int64_t wanted = 4 * (int64_t)simd_count() / waves;
+// arithmetic, so they pay only while whole sequences leave the chip short of waves: `waves` (those that
+// walk whole sequences) must be at most `fill` to a SIMD, and there are as many spans as bring four
+// times that, none shorter than the call's `span`, which its room for the spans' states was sized
+// for.  Measured for 2 x 1,024 tokens (us, whole / cut): the head scan with one wave to a SIMD 309 / 205,
+// with two 327 / 380; the selective scan with half a wave to a SIMD 334 / 176, with one 369 / 311.
+static int span_tokens(int span, int max_count, const float* carry, int64_t waves, int fill) {
+  if (span <= 0 || !carry || waves > (int64_t)fill * simd_count()) return 0;
+  const int64_t wanted = 4 * (int64_t)fill * simd_count() / waves;
   int tokens = (int)((max_count + wanted - 1) / wanted);
   if (tokens < span) tokens = span;
   return max_count >= MIN_SPANS * tokens ? tokens : 0;
@@ -481,7 +481,7 @@ template <typename T, int R>
 static void launch_selective_scan_r(hipStream_t stream, const SelectiveScanCall& c) {
   const int per_token = 2 * 8 * R + 24;
   dim3 block(64);
-  const int span = span_tokens(c.span, c.max_count, c.carry, (int64_t)((c.channels + 7) / 8) * c.n_seqs);
+  const int span = span_tokens(c.span, c.max_count, c.carry, (int64_t)((c.channels + 7) / 8) * c.n_seqs, 2);
   if (span > 0) {
     SelectiveScanCall cut = c;
     cut.span = span;
@@ -557,17 +557,23 @@ struct HeadScanCall {
 // The state of a slot is laid out for this kernel's lanes: [heads][tiles of 4 channels][state][4], so
 // that a wave's load of one register's worth of state (16 state elements by 4 channels) is 256
 // contiguous bytes.  Nobody else reads it; a new sequence's state is all zeros in any layout.
+// A work-group is four waves, each with four channels of the same head: they share the run of B and C in
+// LDS (every wave bringing a quarter of it in) and have one SIMD each.
+#define HS_WAVES 4
+
 template <int R, int PHASE>
-__global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk, int spans) {
+__global__ void __launch_bounds__(64 * HS_WAVES) head_scan_kernel(HeadScanCall c, int chunk, int spans, int tiles) {
   extern __shared__ float lds[];
   constexpr int NP = 16 * R;
   float2* BC = reinterpret_cast<float2*>(lds);                              // [chunk][NP] pairs (B, C): one 8-byte read for both
-  float4* tok = reinterpret_cast<float4*>(lds + (size_t)chunk * NP * 2);    // [chunk][4]: a token and channel's dt * x, D * x, decay, log decay
-  const int lane = threadIdx.x, sub = lane & 15, pl = lane >> 4;
-  const int tile = blockIdx.x, tiles = gridDim.x, head = blockIdx.y;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, sub = lane & 15, pl = lane >> 4;
+  // [waves][chunk][4]: a token and channel's dt * x, D * x, decay, log decay
+  float4* tok = reinterpret_cast<float4*>(lds + (size_t)chunk * NP * 2) + (size_t)wave * chunk * 4;
+  const int tile = min((int)blockIdx.x * HS_WAVES + wave, tiles - 1), head = blockIdx.y;
+  const bool works = (int)blockIdx.x * HS_WAVES + wave < tiles;          // (a wave without a tile only helps to bring B and C in)
   const int seq = blockIdx.z / spans, part = blockIdx.z % spans;
   const int p = tile * 4 + pl;
-  const bool live = p < c.vdim;
+  const bool live = works && p < c.vdim;
   const int group = head / (c.heads / c.groups);
   int first = c.seq_off[seq], last = c.seq_off[seq + 1];
   const int seq_last = last;
@@ -576,7 +582,7 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
   float* mine = nullptr;                             // this span's block of the carry
   if (PHASE) {
     first += part * c.span;
-    if (first >= seq_last) return;
+    if (first >= seq_last) return;                   // (the whole work-group: it is one span's)
     last = min(first + c.span, seq_last);
     mine = c.carry + span_block(c.seq_off, seq, c.span, part) * per_span;
   }
@@ -596,7 +602,7 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
   for (int t0 = first; t0 < last; t0 += chunk) {
     const int count = min(chunk, last - t0);
     __syncthreads();
-    fill_pairs<NP>(BC, Bg, Cg, (int)c.ld, t0, count, c.state, lane);
+    fill_pairs<NP, 64 * HS_WAVES>(BC, Bg, Cg, (int)c.ld, t0, count, c.state, (int)threadIdx.x);
     for (int e = lane; e < count * 4; e += 64) {
       const int i = e >> 2, q = tile * 4 + (e & 3);
       const float xv = q < c.vdim ? c.x[(int64_t)(t0 + i) * c.ld + head * c.vdim + q] : 0.f;
@@ -604,6 +610,7 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
       tok[e] = make_float4(step * xv, Dh * xv, expf(rate * step), rate * step);
     }
     __syncthreads();
+    if (!works) continue;
     // one token: the state moves on; the channel's output (in every lane of its sixteen) is returned
     auto token = [&](int i) -> float {
       const float4 in = tok[i * 4 + pl];
@@ -638,6 +645,7 @@ __global__ void __launch_bounds__(64) head_scan_kernel(HeadScanCall c, int chunk
       if (PHASE != 1 && live && sub == 0) ycol[(int64_t)(t0 + i) * c.ld_y] = y;
     }
   }
+  if (!works) return;
   if (PHASE == 1) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -679,26 +687,26 @@ __global__ void __launch_bounds__(256) head_carry_kernel(HeadScanCall c, int til
 
 template <int R>
 static void launch_head_scan_r(hipStream_t stream, const HeadScanCall& c) {
-  const int per_token = 2 * 16 * R + 16;
-  const int tiles = (c.vdim + 3) / 4;
-  dim3 block(64);
-  const int span = span_tokens(c.span, c.max_count, c.carry, (int64_t)tiles * c.heads * c.n_seqs);
+  const int per_token = 2 * 16 * R + 16 * HS_WAVES;
+  const int tiles = (c.vdim + 3) / 4, groups = (tiles + HS_WAVES - 1) / HS_WAVES;
+  dim3 block(64 * HS_WAVES);
+  const int span = span_tokens(c.span, c.max_count, c.carry, (int64_t)tiles * c.heads * c.n_seqs, 1);
   if (span > 0) {
     HeadScanCall cut = c;
     cut.span = span;
     const int chunk = scan_chunk(per_token, span);
     const int spans = (c.max_count + span - 1) / span;
-    dim3 grid(tiles, c.heads, c.n_seqs * spans);
+    dim3 grid(groups, c.heads, c.n_seqs * spans);
     const size_t lds = (size_t)chunk * per_token * sizeof(float);
-    hipLaunchKernelGGL((head_scan_kernel<R, 1>), grid, block, lds, stream, cut, chunk, spans);
+    hipLaunchKernelGGL((head_scan_kernel<R, 1>), grid, block, lds, stream, cut, chunk, spans, tiles);
     const int64_t size = (int64_t)c.heads * tiles * c.state * 4;
     hipLaunchKernelGGL(head_carry_kernel, dim3((unsigned)((size + 255) / 256), c.n_seqs), dim3(256), 0, stream, cut, tiles);
-    hipLaunchKernelGGL((head_scan_kernel<R, 3>), grid, block, lds, stream, cut, chunk, spans);
+    hipLaunchKernelGGL((head_scan_kernel<R, 3>), grid, block, lds, stream, cut, chunk, spans, tiles);
     return;
   }
   const int chunk = scan_chunk(per_token, c.tokens);
-  dim3 grid(tiles, c.heads, c.n_seqs);
-  hipLaunchKernelGGL((head_scan_kernel<R, 0>), grid, block, (size_t)chunk * per_token * sizeof(float), stream, c, chunk, 1);
+  dim3 grid(groups, c.heads, c.n_seqs);
+  hipLaunchKernelGGL((head_scan_kernel<R, 0>), grid, block, (size_t)chunk * per_token * sizeof(float), stream, c, chunk, 1, tiles);
 }
 
 BT_EXPORT int bt_head_scan_call(void* stream, const HeadScanCall* c) {
