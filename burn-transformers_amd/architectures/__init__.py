@@ -1,3 +1,3 @@
-"""Importing this package registers the architectures the library ships (GPT-2, Salopel)."""
+"""Importing this package registers the architectures the library ships (GPT-2, Salopel, Kodatar)."""
 
-from . import gpt2, salopel  # noqa: F401
+from . import gpt2, kodatar, salopel  # noqa: F401

@@ -57,14 +57,20 @@ RELEASED = -1      # in a sequence's block list: a block behind the group's wind
 class CacheLedger:
     """``windows[g]`` > 0 says that group g only ever reads the last ``windows[g]`` positions of a
     sequence: its blocks that lie wholly behind that window go back to the free list as soon as the
-    sequence has grown past them, and their places in the sequence's list read RELEASED."""
+    sequence has grown past them, and their places in the sequence's list read RELEASED.
+    ``chunks[g]`` > 0 says that a token of group g reads only the positions of its own chunk of that
+    many positions (chunks are counted from position 0): the blocks that lie wholly before the chunk
+    of the next token go back the same way."""
 
-    def __init__(self, n_groups, blocks_per_group, max_slots, max_blocks_per_sequence, windows=None):
+    def __init__(self, n_groups, blocks_per_group, max_slots, max_blocks_per_sequence, windows=None, chunks=None):
         self.n_groups = n_groups
         self.max_blocks_per_sequence = max_blocks_per_sequence
         self.windows = list(windows) if windows is not None else [0] * n_groups
         if len(self.windows) != n_groups or any(w < 0 for w in self.windows):
             raise ValueError(f"{n_groups} groups need {n_groups} windows that are not negative, got {self.windows}")
+        self.chunks = list(chunks) if chunks is not None else [0] * n_groups
+        if len(self.chunks) != n_groups or any(c < 0 for c in self.chunks):
+            raise ValueError(f"{n_groups} groups need {n_groups} chunk sizes that are not negative, got {self.chunks}")
         self.slots = FreeList(max_slots)
         self.blocks = [FreeList(blocks_per_group) for _ in range(n_groups)]
         self.lengths = [0] * max_slots
@@ -101,11 +107,13 @@ class CacheLedger:
 
     def first_kept(self, group, length):
         """Number of the first block of a sequence of ``length`` tokens that group ``group`` still
-        needs: the next token (position ``length``) reads back to position length - window + 1."""
-        window = self.windows[group]
-        if window <= 0:
-            return 0
-        return max(0, length - window + 1) // BLOCK
+        needs: the next token (position ``length``) reads back to position length - window + 1, and
+        not beyond the first position of its chunk."""
+        window, chunk = self.windows[group], self.chunks[group]
+        first = max(0, length - window + 1) if window > 0 else 0
+        if chunk > 0:
+            first = max(first, length - length % chunk)
+        return first // BLOCK
 
     def truncate(self, slot, length):
         """Rewinds a live sequence to ``length`` tokens: the blocks it no longer needs go back
@@ -121,7 +129,7 @@ class CacheLedger:
             held = self.held_blocks[group][slot]
             if RELEASED in held[self.first_kept(group, length):keep]:
                 raise ValueError(f"slot {slot} cannot be rewound to {length} tokens: a layer with a window of "
-                                 f"{self.windows[group]} has given the blocks before it back already")
+                                 f"{self.windows[group]} (or chunks of {self.chunks[group]}) has given the blocks before it back already")
         for group in range(self.n_groups):
             held = self.held_blocks[group][slot]
             while len(held) > keep:
@@ -172,7 +180,7 @@ class CacheLedger:
             raise ValueError(f"slot {slot} cannot shrink from {self.lengths[slot]} to {length}")
         self.lengths[slot] = length
         for group in range(self.n_groups):
-            if self.windows[group] <= 0:
+            if self.windows[group] <= 0 and self.chunks[group] <= 0:
                 continue
             held = self.held_blocks[group][slot]
             for index in range(min(self.first_kept(group, length), len(held))):

@@ -23,10 +23,13 @@ from .ledger import BLOCK, CacheLedger
 @dataclass(frozen=True)
 class KVSpec:
     """What a mixer keeps per token: heads and head size; ``window`` > 0 means that only the last
-    ``window`` positions are ever read."""
+    ``window`` positions are ever read; ``chunk`` > 0 that a token reads only the positions of its own
+    chunk of that many (counted from position 0), so that everything before the chunk the next token
+    falls into is never read again."""
     kv_heads: int
     head_dim: int
     window: int = 0
+    chunk: int = 0
 
 
 @dataclass(frozen=True)
@@ -105,7 +108,8 @@ class Cache:
                 self.state_entry[entry] = (len(self.state_groups), index)
             self.state_groups.append(group)
         self.ledger = CacheLedger(len(self.kv_groups), n_blocks, self.max_slots, self.max_blocks,
-                                  windows=[group.spec.window for group in self.kv_groups])
+                                  windows=[group.spec.window for group in self.kv_groups],
+                                  chunks=[group.spec.chunk for group in self.kv_groups])
 
     # --- slots -----------------------------------------------------------------------------
     def acquire(self):

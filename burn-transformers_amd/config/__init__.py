@@ -1,7 +1,8 @@
 from .base import ConfigError, UnsupportedArchitecture, read_config_json
 from .gpt2 import GPT2Config
+from .kodatar import KodatarConfig
 from .salopel import SalopelConfig
 from .registry import Family, register_family, resolve_family, supported_names, unregister_family
 
-__all__ = ["ConfigError", "UnsupportedArchitecture", "read_config_json", "GPT2Config", "SalopelConfig", "Family",
+__all__ = ["ConfigError", "UnsupportedArchitecture", "read_config_json", "GPT2Config", "KodatarConfig", "SalopelConfig", "Family",
            "register_family", "resolve_family", "supported_names", "unregister_family"]

@@ -29,4 +29,17 @@ struct AttnArgs {
   // Decode (bfloat16 MFMA kernels) only: 0, or `out` is chunk-major with that many rows
   // (activation_offset in common.h); ldo is then not used.
   int out_rows;
+  // 0, or keys are seen in chunks of that many positions, counted from position 0 of the sequence:
+  // a query at position p sees the keys from p - p % chunk through p (and, with a window as well,
+  // only those the window also holds).
+  int chunk;
 };
+
+// The first position a query at `pos` sees: the later of its window's and its chunk's first key.
+// It never decreases as `pos` grows, so the first query of a run of queries has the lowest.
+__host__ __device__ __forceinline__ int bt_first_seen(int pos, int window, int chunk) {
+  int lo = 0;
+  if (window > 0 && pos - window + 1 > lo) lo = pos - window + 1;
+  if (chunk > 0 && pos - pos % chunk > lo) lo = pos - pos % chunk;
+  return lo;
+}

@@ -99,6 +99,7 @@ __device__ __forceinline__ float raise_maximum(float& m, float top, float& alpha
 
 // One tile of 32 keys starting at position kb against NQ tiles of 16 queries.
 //   qpos[nq]: position of the query in column lane % 16 of tile nq, -1 if there is none.
+//   qlo[nq]: the first position that query sees (its window's or its chunk's first key, else 0).
 //   valid_end: positions >= valid_end hold no token (their values are replaced by zero).
 //   c: the score scale times log2(e), positive; m[] is kept in those units (powers of two).
 //   MASKED = false is for tiles every query of the wave sees whole (all keys at or before the
@@ -106,7 +107,7 @@ __device__ __forceinline__ float raise_maximum(float& m, float top, float& alpha
 //   a query then hold numbers nobody reads.
 template <int NQ, bool MASKED>
 __device__ __forceinline__ void attend_tile(const TileOperands& tile, int kb, int valid_end,
-                                            const int (&qpos)[NQ], int window, float c,
+                                            const int (&qpos)[NQ], const int (&qlo)[NQ], float c,
                                             const bf16x8 (&q)[NQ][NKS], floatx4 (&o)[NQ][ND],
                                             float (&m)[NQ], float (&l)[NQ]) {
   const int lane = threadIdx.x & 63, g = lane >> 4;
@@ -127,13 +128,13 @@ __device__ __forceinline__ void attend_tile(const TileOperands& tile, int kb, in
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
     if (MASKED) {
-      const int qp = qpos[nq];
+      const int qp = qpos[nq], ql = qlo[nq];
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           int kp = kb + 16 * t + 4 * g + r;
-          bool seen = kp <= qp && (window == 0 || kp > qp - window);
+          bool seen = kp <= qp && kp >= ql;
           s[nq][t][r] = seen ? s[nq][t][r] : -INFINITY;
         }
     }
@@ -261,7 +262,7 @@ attention_prefill_kernel(AttnArgs a) {
   const bf16_t* Q = static_cast<const bf16_t*>(a.q);
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  int qpos[PREFILL_NQ], tok[PREFILL_NQ];
+  int qpos[PREFILL_NQ], qlo[PREFILL_NQ], tok[PREFILL_NQ];
   bf16x8 q[PREFILL_NQ][NKS];
   floatx4 o[PREFILL_NQ][ND];
   float m[PREFILL_NQ], l[PREFILL_NQ];
@@ -270,6 +271,7 @@ attention_prefill_kernel(AttnArgs a) {
     int qi = q0 + nq * 16 + i16;
     bool exists = qi < count;
     qpos[nq] = exists ? start + qi : -1;
+    qlo[nq] = exists ? bt_first_seen(start + qi, a.window, a.chunk) : 0;
     tok[nq] = off + (exists ? qi : count - 1);
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
@@ -283,8 +285,7 @@ attention_prefill_kernel(AttnArgs a) {
   }
   const int last = q0 + PREFILL_QUERIES_PER_WAVE < count ? q0 + PREFILL_QUERIES_PER_WAVE : count;
   const int hi = start + last;  // one past the position of this wave's last query
-  int lo = 0;
-  if (a.window > 0 && start + q0 - a.window + 1 > 0) lo = (start + q0 - a.window + 1) & ~31;
+  const int lo = bt_first_seen(start + q0, a.window, a.chunk) & ~31;      // (the wave's first query sees furthest back)
   const int valid_end = start + count;
   const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
   const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
@@ -292,7 +293,7 @@ attention_prefill_kernel(AttnArgs a) {
   // is copied: while one is multiplied the other is in flight.  (A third set, two tiles ahead,
   // costs the registers that let two work-groups share a compute unit, and measured slower.)
   const float c = a.scale * LOG2_E;
-  const int whole_until = a.window == 0 ? start + q0 + 1 : 0;   // tiles ending here or before are seen whole
+  const int whole_until = a.window == 0 && a.chunk == 0 ? start + q0 + 1 : 0;   // tiles ending here or before are seen whole
   // A fetch beyond the last tile reads the first one again instead of being skipped: with the same
   // number of loads in flight on every path, the wait before a tile is for that tile only.
   TileOperands t0, t1;
@@ -303,9 +304,9 @@ attention_prefill_kernel(AttnArgs a) {
   };
   auto attend = [&](const TileOperands& tile, int kb) {
     if (kb + 32 <= whole_until)
-      attend_tile<PREFILL_NQ, false>(tile, kb, valid_end, qpos, a.window, c, q, o, m, l);
+      attend_tile<PREFILL_NQ, false>(tile, kb, valid_end, qpos, qlo, c, q, o, m, l);
     else
-      attend_tile<PREFILL_NQ, true>(tile, kb, valid_end, qpos, a.window, c, q, o, m, l);
+      attend_tile<PREFILL_NQ, true>(tile, kb, valid_end, qpos, qlo, c, q, o, m, l);
   };
   if (lo >= hi) return;   // (cannot happen: a wave with a query sees at least that query's key)
   fetch(t0, lo);
@@ -756,7 +757,7 @@ attention_decode_kernel(AttnArgs a) {
   const int* block_row = a.kv.blocks + (int64_t)seq * a.kv.max_blocks;
   const int last_entry = a.kv.max_blocks - 1;
   int early_block0 = 0, early_block1 = 0;
-  const bool early = a.window == 0 && splits == 1;    // (a later run's first tiles depend on the position)
+  const bool early = a.window == 0 && a.chunk == 0 && splits == 1;    // (a later run's first tiles depend on the position)
   if (early) {
     int entry0 = (32 * wave) / BT_KV_BLOCK, entry1 = (32 * wave + stride) / BT_KV_BLOCK;
     early_block0 = block_row[entry0 < last_entry ? entry0 : last_entry];
@@ -770,13 +771,13 @@ attention_decode_kernel(AttnArgs a) {
     q[0][ks] = (has_query && channel < HD) ? load_bf16x8(Q + (int64_t)tok * a.ldq + head * HD + channel) : zero8;
   }
   int qpos[1] = {has_query ? pos : -1};
+  const int qlo[1] = {bt_first_seen(pos, a.window, a.chunk)};
   floatx4 o[1][ND];
   float m[1] = {-INFINITY}, l[1] = {0.f};
 #pragma unroll
   for (int dt = 0; dt < ND; ++dt) o[0][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  int lo = 0;
-  if (a.window > 0 && pos - a.window + 1 > 0) lo = (pos - a.window + 1) & ~31;
+  const int lo = qlo[0] & ~31;
   const bf16_t* keys = static_cast<const bf16_t*>(a.kv.keys);
   const bf16_t* values = static_cast<const bf16_t*>(a.kv.values);
   // the tiles of 32 keys from `lo` through the query's own position, cut into `splits` runs
@@ -797,7 +798,7 @@ attention_decode_kernel(AttnArgs a) {
     }
   };
   auto attend = [&](const TileOperands& tile, int kb) {   // one form: this kernel waits for memory, not for the ALU
-    attend_tile<1, true>(tile, kb, pos + 1, qpos, a.window, c, q, o, m, l);
+    attend_tile<1, true>(tile, kb, pos + 1, qpos, qlo, c, q, o, m, l);
   };
   TileOperands current, next;
   fetch(next, first, 0);
@@ -910,7 +911,7 @@ static int check_args(const AttnArgs& a, const char* who) {
   if (a.kv.head_dim != HD) BT_REFUSE("%s: built for head size %d, asked for %d", who, HD, a.kv.head_dim);
   if (a.kv.kv_heads <= 0 || a.q_heads <= 0 || a.q_heads % a.kv.kv_heads != 0)
     BT_REFUSE("%s: %d query heads cannot share %d key/value heads", who, a.q_heads, a.kv.kv_heads);
-  if (a.window < 0) BT_REFUSE("%s: window %d must not be negative", who, a.window);
+  if (a.window < 0 || a.chunk < 0) BT_REFUSE("%s: window %d and chunk %d must not be negative", who, a.window, a.chunk);
   if (!(a.scale > 0.f)) BT_REFUSE("%s: the score scale %g must be positive (the maximum is taken before scaling)", who, a.scale);
   if (!a.q || !a.out || !a.seq_off || !a.seq_start || !a.kv.blocks || !a.kv.keys || !a.kv.values)
     BT_REFUSE("%s: missing operand", who);
@@ -928,7 +929,7 @@ BT_EXPORT int bt_attention_prefill_bf16(void* stream, const AttnArgs* args) {
   if (rc) return rc;
   if (args->max_count <= 0) BT_REFUSE("attention_prefill_bf16: max_count %d must be positive", args->max_count);
   const int runs = args->splits > 1 ? args->splits : 1;
-  if (runs > 1 && (HD != 64 || args->window != 0 || !args->partial || runs > 64))
+  if (runs > 1 && (HD != 64 || args->window != 0 || args->chunk != 0 || !args->partial || runs > 64))
     BT_REFUSE("attention_prefill_bf16: runs of keys (%d) are for heads of 64 without a window, at most 64, and need a place "
               "for their partial results", runs);
   const int q_tiles = (args->max_count + PREFILL_QUERIES - 1) / PREFILL_QUERIES;
@@ -947,7 +948,7 @@ BT_EXPORT int bt_attention_prefill_bf16(void* stream, const AttnArgs* args) {
   if (groups > 0x7fffffff) BT_REFUSE("attention_prefill_bf16: %lld work-groups are too many", (long long)groups);
   dim3 grid((unsigned)groups);
 #if BT_HEAD_DIM == 64
-  if (args->window == 0) {   // keys and values shared through LDS, a tile's keys on two sets of waves
+  if (args->window == 0 && args->chunk == 0) {   // keys and values shared through LDS, a tile's keys on two sets of waves
     static bool raised = false;                 // 72 KB: beyond what a kernel gets without asking
     if (!raised) {
       hipError_t err = hipFuncSetAttribute((const void*)attention_prefill_split_kernel,

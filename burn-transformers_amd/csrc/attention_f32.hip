@@ -61,16 +61,18 @@ attention_f32_mfma_kernel(AttnArgs a) {
   const int i16 = lane & 15, g = lane >> 4;
   const int n_queries = count - q0 < F32M_QUERIES ? count - q0 : F32M_QUERIES;
   const int first_pos = start + q0, last_pos = first_pos + n_queries - 1;
-  const int lo_pos = (a.window > 0 && first_pos - a.window + 1 > 0) ? first_pos - a.window + 1 : 0;
+  const int lo_pos = bt_first_seen(first_pos, a.window, a.chunk);
   const int first_block = lo_pos / BT_KV_BLOCK, last_block = last_pos / BT_KV_BLOCK;
   const bool wave_active = wave * 16 < n_queries;
   // what the wave's queries can see at all: positions wave_lo .. wave_hi
   const int wave_first = first_pos + wave * 16;
   const int wave_hi = wave_first + 15 < last_pos ? wave_first + 15 : last_pos;
-  const int wave_lo = (a.window > 0 && wave_first - a.window + 1 > 0) ? wave_first - a.window + 1 : 0;
+  const int wave_lo = bt_first_seen(wave_first, a.window, a.chunk);
+  const int wave_hi_lo = bt_first_seen(wave_hi, a.window, a.chunk);   // the first key that its last query sees
   const int mine = wave * 16 + i16;                          // the lane's query within the tile
   const bool exists = wave_active && mine < n_queries;
   const int qpos = exists ? first_pos + mine : -1;           // (a column without a query sees no key and is never stored)
+  const int qlo = exists ? bt_first_seen(qpos, a.window, a.chunk) : 0;
 
   const float* q = static_cast<const float*>(a.q);
   floatx4 qreg[KS];
@@ -153,14 +155,14 @@ attention_f32_mfma_kernel(AttnArgs a) {
 #pragma unroll
     for (int dt = 0; dt < KS; ++dt) v4[0][dt] = *reinterpret_cast<const floatx4*>(vcol + 64 * dt);
     // a block that every query of the wave sees whole needs no comparisons
-    const bool whole = kb + BT_KV_BLOCK - 1 <= wave_first && (a.window <= 0 || kb > wave_hi - a.window);
+    const bool whole = kb + BT_KV_BLOCK - 1 <= wave_first && kb >= wave_hi_lo;
     if (!whole) {
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key_pos = kb + 16 * t + 4 * g + r;
-          const bool seen = key_pos <= qpos && (a.window <= 0 || key_pos > qpos - a.window);
+          const bool seen = key_pos <= qpos && key_pos >= qlo;
           s[t][r] = seen ? s[t][r] : -INFINITY;
         }
     }
@@ -236,7 +238,7 @@ attention_f32_decode_kernel(AttnArgs a) {
   const float* q = static_cast<const float*>(a.q) + (int64_t)seq * a.ldq + head * hd;
   if (tid < hd) qs[tid] = q[tid];
   __syncthreads();
-  const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+  const int lo = bt_first_seen(pos, a.window, a.chunk);
   int first_block = lo / BT_KV_BLOCK, last_block = pos / BT_KV_BLOCK;
   const int splits = a.splits > 1 ? a.splits : 1, split = blockIdx.z;
   if (splits > 1) {       // this work-group's run of the blocks (it may be empty)
@@ -388,7 +390,7 @@ BT_EXPORT int bt_attention_f32(void* stream, const AttnArgs* args) {
   if (hd <= 0 || hd % 16 != 0 || hd > 128) BT_REFUSE("attention_f32: head size %d must be a multiple of 16 up to 128", hd);
   if (a.kv.kv_heads <= 0 || a.q_heads <= 0 || a.q_heads % a.kv.kv_heads != 0)
     BT_REFUSE("attention_f32: %d query heads cannot share %d key/value heads", a.q_heads, a.kv.kv_heads);
-  if (a.window < 0) BT_REFUSE("attention_f32: window %d must not be negative", a.window);
+  if (a.window < 0 || a.chunk < 0) BT_REFUSE("attention_f32: window %d and chunk %d must not be negative", a.window, a.chunk);
   if (a.max_count <= 0) BT_REFUSE("attention_f32: max_count %d must be positive", a.max_count);
   if (!(a.scale > 0.f)) BT_REFUSE("attention_f32: scale %g must be positive", (double)a.scale);
   if (!a.q || !a.out || !a.seq_off || !a.seq_start || !a.kv.blocks || !a.kv.keys || !a.kv.values)

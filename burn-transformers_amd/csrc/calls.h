@@ -30,6 +30,8 @@ struct EmbedCall {
   const void* table;
   const void* positions;   // or null
   float* out;
+  float scale;             // multiplies the token's row (not the position's)
+  float* copy;             // or null: a second place for the same rows
 };
 
 struct AddNormCall {

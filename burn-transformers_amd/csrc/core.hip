@@ -20,33 +20,35 @@
 #include "no_alloc.h"
 
 // ---------------------------------------------------------------------------------------------
-// Embedding: x[t] = table[ids[t]] (+ positions[pos[t]]), written as 32-bit residual stream.
+// Embedding: x[t] = scale * table[ids[t]] (+ positions[pos[t]]), written as 32-bit residual stream
+// (and, where a model reads the embedding's output again later, to a second place as well).
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ pos,
                              const T* __restrict__ table, const T* __restrict__ positions,
-                             float* __restrict__ out, int width) {
+                             float* __restrict__ out, float* __restrict__ copy, float scale, int width) {
   int t = blockIdx.x;
   const T* row = table + (int64_t)ids[t] * width;
   const T* prow = positions ? positions + (int64_t)pos[t] * width : nullptr;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
-    float v = to_float(row[c]);
+    float v = to_float(row[c]) * scale;
     if (prow) v += to_float(prow[c]);
     out[(int64_t)t * width + c] = v;
+    if (copy) copy[(int64_t)t * width + c] = v;
   }
 }
 
 BT_EXPORT int bt_embed(void* stream, int dtype, const int* ids, const int* pos, const void* table,
-                       const void* positions, float* out, int tokens, int width) {
+                       const void* positions, float* out, int tokens, int width, float scale, float* copy) {
   if (tokens <= 0) return BT_OK;
   if (width <= 0) BT_REFUSE("embed: width %d must be positive", width);
   dim3 grid(tokens), block(256);
   if (dtype == 0)
     hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, (hipStream_t)stream, ids, pos,
-                       (const float*)table, (const float*)positions, out, width);
+                       (const float*)table, (const float*)positions, out, copy, scale, width);
   else
     hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, ids, pos,
-                       (const bf16_t*)table, (const bf16_t*)positions, out, width);
+                       (const bf16_t*)table, (const bf16_t*)positions, out, copy, scale, width);
   return bt_check_launch("embed");
 }
 
@@ -450,7 +452,8 @@ BT_EXPORT int bt_gemm_plain(void* stream, int dtype, const void* A, int64_t lda,
 
 // ---------------------------------------------------------------------------------------------
 // Plain attention over the paged cache.  One work-group per (token, query head).
-//   scores s_k = scale * (q . key_k) for keys lo <= k <= pos, lo = max(0, pos - window + 1)
+//   scores s_k = scale * (q . key_k) for keys lo <= k <= pos, lo = max(0, pos - window + 1), or the
+//   first position of pos's chunk if that is later (bt_first_seen)
 //   out = sum_k softmax(s)_k value_k, softmax in 32-bit with a running maximum over chunks.
 // Keys beyond the token's own position are never read.
 // ---------------------------------------------------------------------------------------------
@@ -471,7 +474,7 @@ attention_plain_kernel(AttnArgs a) {
   const T* q = static_cast<const T*>(a.q) + (int64_t)t * a.ldq + head * hd;
   for (int c = threadIdx.x; c < hd; c += blockDim.x) qs[c] = to_float(q[c]);
   __syncthreads();
-  int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+  int lo = bt_first_seen(pos, a.window, a.chunk);
   float run_max = -INFINITY, run_sum = 0.f, acc = 0.f;  // acc: channel threadIdx.x (< hd)
   const T* keys = static_cast<const T*>(a.kv.keys);
   const T* values = static_cast<const T*>(a.kv.values);
@@ -522,7 +525,7 @@ int bt_check_attention(const AttnArgs& a, const char* who) {
   if (hd <= 0 || hd > 256) BT_REFUSE("%s: head size %d outside 1..256 (a work-group holds a query and one channel per thread)", who, hd);
   if (a.kv.kv_heads <= 0 || a.q_heads <= 0 || a.q_heads % a.kv.kv_heads != 0)
     BT_REFUSE("%s: %d query heads cannot share %d key/value heads", who, a.q_heads, a.kv.kv_heads);
-  if (a.window < 0) BT_REFUSE("%s: window %d must not be negative", who, a.window);
+  if (a.window < 0 || a.chunk < 0) BT_REFUSE("%s: window %d and chunk %d must not be negative", who, a.window, a.chunk);
   if (!a.q || !a.out || !a.tok_seq || !a.tok_pos || !a.seq_off || !a.seq_start || !a.kv.blocks ||
       !a.kv.keys || !a.kv.values)
     BT_REFUSE("%s: missing operand", who);
@@ -1241,7 +1244,7 @@ BT_EXPORT int bt_count_tokens(void* stream, int* counts, int64_t ld, const int* 
 // The same entry points with their arguments as one structure (calls.h), for launch lists.
 // ---------------------------------------------------------------------------------------------
 BT_EXPORT int bt_embed_call(void* stream, const EmbedCall* c) {
-  return bt_embed(stream, c->dtype, c->ids, c->pos, c->table, c->positions, c->out, c->tokens, c->width);
+  return bt_embed(stream, c->dtype, c->ids, c->pos, c->table, c->positions, c->out, c->tokens, c->width, c->scale, c->copy);
 }
 BT_EXPORT int bt_add_norm_call(void* stream, const AddNormCall* c) {
   return bt_add_norm(stream, c->out_dtype, c->x, c->delta, c->n_delta, c->delta_stride, c->bias, c->gamma, c->beta, c->eps,

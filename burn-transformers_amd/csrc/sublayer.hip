@@ -1,7 +1,9 @@
 // Kernels for layers that normalise a sublayer's OUTPUT before it joins the residual stream, and
 // for activations that are norms themselves.  All statistics and the residual sum are 32-bit.
-//   * output norm: x[t] (+)= mult * v / sqrt(mean(v^2) + eps) * gamma, v the sublayer's output
-//     (the sum of its partial sums and its bias), and a copy of the new x in the products' type
+//   * output norm: x[t] (+)= mult * N(v), v the sublayer's output (the sum of its partial sums and
+//     its bias), N an RMS norm, v / sqrt(mean(v^2) + eps) * gamma, or a layer norm,
+//     (v - mean) / sqrt(var + eps) * gamma + beta; and a copy of the new x in the products' type
+//   * joined rows: [x | y] side by side in the products' type, the operand of a product that reads two streams
 //   * PolyNorm: a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over a row
 #include "host.h"
 
@@ -22,6 +24,8 @@ struct OutputNormCall {
   const float* gamma;    // [width]
   void* cast;            // [tokens][ld_cast] or null
   int64_t ld_cast;
+  int kind;              // 0: layer norm (mean taken off, `beta` added), 1: RMS norm
+  const float* beta;     // [width] or null
 };
 
 template <typename T>
@@ -40,13 +44,20 @@ __global__ void __launch_bounds__(256) output_norm_kernel(OutputNormCall c) {
       for (int s = 0; s < c.n_delta; ++s) v += c.delta[s * c.delta_stride + (int64_t)t * c.ldd + col];
     }
     row_buf[col] = v;
-    partial += v * v;
+    partial += v;
+  }
+  const float mean = c.kind == 0 ? block_sum(partial, scratch) / (float)c.width : 0.f;
+  partial = 0.f;
+  for (int col = threadIdx.x; col < c.width; col += blockDim.x) {
+    const float d = row_buf[col] - mean;
+    partial += d * d;
   }
   const float total = block_sum(partial, scratch);
   const float scale = c.mult / sqrtf(total / (float)c.width + c.eps);
   T* cast = static_cast<T*>(c.cast);
   for (int col = threadIdx.x; col < c.width; col += blockDim.x) {
-    float y = row_buf[col] * scale * c.gamma[col];
+    float y = (row_buf[col] - mean) * scale * c.gamma[col];
+    if (c.beta) y += c.mult * c.beta[col];
     if (c.accumulate) y += xr[col];
     xr[col] = y;
     if (cast) cast[(int64_t)t * c.ld_cast + col] = from_float<T>(y);
@@ -64,13 +75,14 @@ __global__ void __launch_bounds__(256) output_norm_small_kernel(OutputNormCall c
   __shared__ float scratch[32];
   const int t = blockIdx.x;
   float* xr = c.x + (int64_t)t * c.width;
-  float v[KMAX], xv[KMAX], g[KMAX];
+  float v[KMAX], xv[KMAX], g[KMAX], b[KMAX];
 #pragma unroll
   for (int k = 0; k < KMAX; ++k) {
     const int col = threadIdx.x + 256 * k;
-    v[k] = xv[k] = g[k] = 0.f;
+    v[k] = xv[k] = g[k] = b[k] = 0.f;
     if (col < c.width) {
       g[k] = c.gamma[col];
+      if (c.beta) b[k] = c.mult * c.beta[col];
       if (c.n_delta == 0) {
         v[k] = xr[col];
       } else {
@@ -82,6 +94,14 @@ __global__ void __launch_bounds__(256) output_norm_small_kernel(OutputNormCall c
     }
   }
   float partial = 0.f;
+  if (c.kind == 0) {          // a layer norm: the mean first, then the squared distances from it
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) partial += v[k];
+    const float mean = block_sum(partial, scratch) / (float)c.width;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) v[k] = threadIdx.x + 256 * k < c.width ? v[k] - mean : 0.f;
+    partial = 0.f;
+  }
 #pragma unroll
   for (int k = 0; k < KMAX; ++k) partial += v[k] * v[k];
   const float scale = c.mult / sqrtf(block_sum(partial, scratch) / (float)c.width + c.eps);
@@ -90,7 +110,7 @@ __global__ void __launch_bounds__(256) output_norm_small_kernel(OutputNormCall c
   for (int k = 0; k < KMAX; ++k) {
     const int col = threadIdx.x + 256 * k;
     if (col < c.width) {
-      const float y = v[k] * scale * g[k] + xv[k];
+      const float y = v[k] * scale * g[k] + b[k] + xv[k];
       xr[col] = y;
       if (cast) cast[(int64_t)t * c.ld_cast + col] = from_float<T>(y);
     }
@@ -116,6 +136,7 @@ BT_EXPORT int bt_output_norm_call(void* stream, const OutputNormCall* c) {
   if (c->width <= 0 || c->width > 15360) BT_REFUSE("output_norm: width %d outside 1..15360", c->width);
   if (!c->x || !c->gamma || (c->n_delta > 0 && !c->delta)) BT_REFUSE("output_norm: missing operand");
   if (c->n_delta == 0 && c->accumulate) BT_REFUSE("output_norm: the stream's own rows cannot be added to themselves");
+  if (c->kind != 0 && c->kind != 1) BT_REFUSE("output_norm: unknown kind of norm %d", c->kind);
   if (c->cast && (c->cast_cols < c->width || c->ld_cast < c->cast_cols))
     BT_REFUSE("output_norm: a copy of %d columns in rows of %lld does not hold width %d", c->cast_cols,
               (long long)c->ld_cast, c->width);
@@ -124,6 +145,43 @@ BT_EXPORT int bt_output_norm_call(void* stream, const OutputNormCall* c) {
   else
     launch_output_norm<bf16_t>((hipStream_t)stream, *c);
   return bt_check_launch("output_norm");
+}
+
+// out[t] = [x[t] | y[t] | zeros] in the products' type: the operand of a product over two float32
+// streams laid side by side (W [x; y] as one product).
+struct JoinRowsCall {
+  int out_dtype;         // 0 float32, 1 bfloat16
+  int tokens;
+  int width;             // columns of x and of y
+  int out_cols;          // columns of out written: 2 * width, then zeros
+  const float* x;        // [tokens][width]
+  const float* y;        // [tokens][width]
+  void* out;             // [tokens][ldo]
+  int64_t ldo;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) join_rows_kernel(JoinRowsCall c) {
+  const int t = blockIdx.x;
+  T* out = static_cast<T*>(c.out) + (int64_t)t * c.ldo;
+  for (int col = threadIdx.x; col < c.out_cols; col += blockDim.x) {
+    float v = 0.f;
+    if (col < c.width) v = c.x[(int64_t)t * c.width + col];
+    else if (col < 2 * c.width) v = c.y[(int64_t)t * c.width + col - c.width];
+    out[col] = from_float<T>(v);
+  }
+}
+
+BT_EXPORT int bt_join_rows_call(void* stream, const JoinRowsCall* c) {
+  if (c->tokens <= 0) return BT_OK;
+  if (c->width <= 0 || c->out_cols < 2 * c->width || c->ldo < c->out_cols)
+    BT_REFUSE("join_rows: rows of %lld columns (%d written) do not hold two of width %d", (long long)c->ldo, c->out_cols, c->width);
+  if (!c->x || !c->y || !c->out) BT_REFUSE("join_rows: missing operand");
+  if (c->out_dtype == 0)
+    hipLaunchKernelGGL(join_rows_kernel<float>, dim3(c->tokens), dim3(256), 0, (hipStream_t)stream, *c);
+  else
+    hipLaunchKernelGGL(join_rows_kernel<bf16_t>, dim3(c->tokens), dim3(256), 0, (hipStream_t)stream, *c);
+  return bt_check_launch("join_rows");
 }
 
 struct PolyNormCall {

@@ -48,7 +48,7 @@ class AttnArgs(ctypes.Structure):
                 ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("seq_off", _c_ptr), ("seq_start", _c_ptr),
                 ("kv", KvView), ("q_heads", _c_int), ("n_tokens", _c_int), ("n_seqs", _c_int),
                 ("max_count", _c_int), ("window", _c_int), ("scale", _c_float), ("splits", _c_int),
-                ("partial", _c_ptr), ("out_rows", _c_int)]
+                ("partial", _c_ptr), ("out_rows", _c_int), ("chunk", _c_int)]
 
 
 class NormOperand(ctypes.Structure):
@@ -58,7 +58,7 @@ class NormOperand(ctypes.Structure):
 
 class EmbedCall(ctypes.Structure):
     _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("width", _c_int), ("ids", _c_ptr), ("pos", _c_ptr),
-                ("table", _c_ptr), ("positions", _c_ptr), ("out", _c_ptr)]
+                ("table", _c_ptr), ("positions", _c_ptr), ("out", _c_ptr), ("scale", _c_float), ("copy", _c_ptr)]
 
 
 class AddNormCall(ctypes.Structure):
@@ -87,7 +87,13 @@ class OutputNormCall(ctypes.Structure):
     _fields_ = [("cast_dtype", _c_int), ("n_delta", _c_int), ("tokens", _c_int), ("width", _c_int),
                 ("accumulate", _c_int), ("cast_cols", _c_int), ("eps", _c_float), ("mult", _c_float), ("x", _c_ptr),
                 ("delta", _c_ptr), ("delta_stride", _c_i64), ("ldd", _c_i64), ("bias", _c_ptr), ("gamma", _c_ptr),
-                ("cast", _c_ptr), ("ld_cast", _c_i64)]
+                ("cast", _c_ptr), ("ld_cast", _c_i64), ("kind", _c_int), ("beta", _c_ptr)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class JoinRowsCall(ctypes.Structure):
+    _fields_ = [("out_dtype", _c_int), ("tokens", _c_int), ("width", _c_int), ("out_cols", _c_int), ("x", _c_ptr),
+                ("y", _c_ptr), ("out", _c_ptr), ("ldo", _c_i64)]
     _step_fields_ = {"tokens": "tokens"}
 
 
@@ -148,6 +154,29 @@ class GatedNormCall(ctypes.Structure):
     _fields_ = [("out_dtype", _c_int), ("tokens", _c_int), ("channels", _c_int), ("parts", _c_int), ("out_cols", _c_int),
                 ("eps", _c_float), ("y", _c_ptr), ("ld_y", _c_i64), ("z", _c_ptr), ("ld_z", _c_i64), ("weight", _c_ptr),
                 ("out", _c_ptr), ("ld_out", _c_i64)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class HeadRotaryCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("heads", _c_int), ("kv_heads", _c_int), ("dim", _c_int),
+                ("vdim", _c_int), ("rot_dims", _c_int), ("eps", _c_float), ("input", _c_ptr), ("ld", _c_i64),
+                ("q_gamma", _c_ptr), ("k_gamma", _c_ptr), ("inv_freq", _c_ptr), ("q_out", _c_ptr), ("ld_q", _c_i64),
+                ("tok_seq", _c_ptr), ("tok_pos", _c_ptr), ("kv", KvView)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class RouteCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("width", _c_int), ("experts", _c_int), ("top", _c_int),
+                ("groups", _c_int), ("keep", _c_int), ("h", _c_ptr), ("ldh", _c_i64), ("W", _c_ptr),
+                ("correction", _c_ptr), ("gate_w", _c_ptr), ("weights", _c_ptr), ("gate", _c_ptr)]
+    _step_fields_ = {"tokens": "tokens"}
+
+
+class GatedExpertsCall(ctypes.Structure):
+    _fields_ = [("dtype", _c_int), ("tokens", _c_int), ("experts", _c_int), ("ff", _c_int), ("shared_ff", _c_int),
+                ("identity", _c_int), ("hidden_cols", _c_int), ("width", _c_int), ("gu", _c_ptr), ("ld_gu", _c_i64),
+                ("weights", _c_ptr), ("gate", _c_ptr), ("hidden", _c_ptr), ("ld_hidden", _c_i64), ("h", _c_ptr),
+                ("ldh", _c_i64), ("identity_out", _c_ptr)]
     _step_fields_ = {"tokens": "tokens"}
 
 
@@ -592,11 +621,13 @@ def epilogue_qkv(q_out, n_q, n_kv, kv_view, tok_seq, tok_pos, bias=None):
 
 # --- kernels ---------------------------------------------------------------------------------
 
-def embed(ids, positions, table, position_table, out):
-    """out[t] = table[ids[t]] (+ position_table[positions[t]]); out is the float32 stream."""
+def embed(ids, positions, table, position_table, out, scale=1.0, copy=None):
+    """out[t] = scale * table[ids[t]] (+ position_table[positions[t]]); out is the float32 stream,
+    ``copy`` an optional second float32 place for the same rows."""
     _launch(_module("core"), "bt_embed_call",
             EmbedCall(dtype=DTYPE_CODES[table.dtype], tokens=ids.numel(), width=table.shape[1], ids=ids.data_ptr(),
-                      pos=_ptr(positions), table=table.data_ptr(), positions=_ptr(position_table), out=out.data_ptr()))
+                      pos=_ptr(positions), table=table.data_ptr(), positions=_ptr(position_table), out=out.data_ptr(),
+                      scale=scale, copy=_ptr(copy)))
 
 
 def add_norm(x, out, gamma, beta, eps, kind="layer_norm", delta=None, bias=None, rows=None,
@@ -833,12 +864,14 @@ def _library_has_algorithm(lda, m, n, k, epilogue):
 
 
 def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_heads, n_seqs, max_count,
-                   scale, window=0, partial=None, runs=None):
+                   scale, window=0, partial=None, runs=None, chunk=0):
     """``partial``: float32 [rows * q_heads * runs, head_dim + 2] for a step whose keys are cut into
     runs that separate work-groups take.  Decode steps (long contexts in small batches): rows are
     the sequences, and ``runs`` follows from the shape.  Prompt steps (few query tiles behind a long
     context): rows are the step's tokens, the buffer may be longer than this step needs, and
-    ``runs`` is given.  ``out`` may be a :class:`Chunked` for the bfloat16 decode kernels."""
+    ``runs`` is given.  ``out`` may be a :class:`Chunked` for the bfloat16 decode kernels.
+    ``chunk`` > 0: a query at position p sees only the keys from p - p % chunk on (chunks are counted
+    from position 0 of its sequence); ``window`` > 0: only the last ``window`` positions."""
     splits = 1
     if partial is not None:
         rows = n_seqs if runs is None else q.shape[0]
@@ -851,7 +884,7 @@ def attention_args(q, out, kv_view, tok_seq, tok_pos, seq_off, seq_start, q_head
                     q=q.data_ptr(), ldq=q.stride(0), out=out.data_ptr(), ldo=out.stride(0), out_rows=_out_rows(out),
                     tok_seq=tok_seq.data_ptr(), tok_pos=tok_pos.data_ptr(), seq_off=seq_off.data_ptr(),
                     seq_start=seq_start.data_ptr(), kv=kv_view, q_heads=q_heads, n_tokens=q.shape[0],
-                    n_seqs=n_seqs, max_count=max_count, window=window or 0, scale=scale)
+                    n_seqs=n_seqs, max_count=max_count, window=window or 0, scale=scale, chunk=chunk or 0)
 
 
 def attention(args, dtype, decode, impl="auto"):
@@ -971,10 +1004,11 @@ def count_tokens(counts, rows, tokens):
 
 # --- norms of a sublayer's output, activations that are norms ---------------------------------
 
-def output_norm(x, gamma, eps, mult=1.0, delta=None, bias=None, accumulate=True, cast=None):
-    """x[t] (+)= mult * v / sqrt(mean(v^2) + eps) * gamma with v = sum(delta[:, t]) + bias (``delta``
-    float32 [splits, tokens, width] or [tokens, width]); without ``delta`` the stream's own rows are
-    normalised in place (``accumulate`` must then be False).  ``cast``: a tensor [tokens, >= width]
+def output_norm(x, gamma, eps, mult=1.0, delta=None, bias=None, accumulate=True, cast=None, kind="rms_norm", beta=None):
+    """x[t] (+)= mult * N(v) with v = sum(delta[:, t]) + bias (``delta`` float32 [splits, tokens, width]
+    or [tokens, width]) and N the norm of ``kind``: v / sqrt(mean(v^2) + eps) * gamma, or for
+    "layer_norm" (v - mean) / sqrt(var + eps) * gamma + beta; without ``delta`` the stream's own rows
+    are normalised in place (``accumulate`` must then be False).  ``cast``: a tensor [tokens, >= width]
     in the products' type that receives the new x (and zeros behind it)."""
     tokens, width = x.shape
     if delta is None:
@@ -988,7 +1022,16 @@ def output_norm(x, gamma, eps, mult=1.0, delta=None, bias=None, accumulate=True,
                            tokens=tokens, width=width, accumulate=1 if accumulate else 0,
                            cast_cols=cast.shape[1] if cast is not None else 0, eps=eps, mult=mult, x=x.data_ptr(),
                            delta=_ptr(delta), delta_stride=stride, ldd=ldd, bias=_ptr(bias), gamma=gamma.data_ptr(),
-                           cast=_ptr(cast), ld_cast=cast.stride(0) if cast is not None else 0))
+                           cast=_ptr(cast), ld_cast=cast.stride(0) if cast is not None else 0,
+                           kind=NORM_KINDS[kind], beta=_ptr(beta)))
+
+
+def join_rows(x, y, out):
+    """out[t] = [x[t] | y[t] | zeros]: two float32 streams [tokens, width] side by side in the products'
+    type, the operand of one product over both."""
+    _launch(_module("sublayer"), "bt_join_rows_call",
+            JoinRowsCall(out_dtype=DTYPE_CODES[out.dtype], tokens=x.shape[0], width=x.shape[1], out_cols=out.shape[1],
+                         x=x.data_ptr(), y=y.data_ptr(), out=out.data_ptr(), ldo=out.stride(0)))
 
 
 def poly_norm(z, columns, coefficients, eps, out):
@@ -1105,3 +1148,47 @@ def gated_norm(y, z, weight, parts, eps, out):
             GatedNormCall(out_dtype=DTYPE_CODES[out.dtype], tokens=y.shape[0], channels=weight.shape[0], parts=parts,
                           out_cols=out.shape[1], eps=eps, y=y.data_ptr(), ld_y=y.stride(0), z=z.data_ptr(),
                           ld_z=z.stride(0), weight=weight.data_ptr(), out=out.data_ptr(), ld_out=out.stride(0)))
+
+
+# --- rotary positions -------------------------------------------------------------------------
+
+def head_rotary(fused, heads, kv_heads, dim, vdim, rot_dims, inv_freq, q_gamma, k_gamma, eps, q_out, tok_seq, tok_pos,
+                kv_view, dtype):
+    """Behind a fused query/key/value projection with float32 rows ``fused`` (queries heads * dim, keys
+    kv_heads * dim, values kv_heads * vdim): every query and key head divided by its root mean square
+    times ``q_gamma`` / ``k_gamma`` ([dim] float32; None: no norm), the first ``rot_dims`` channels of each
+    turned by the token's position (channel i with i + rot_dims / 2, angle position * ``inv_freq[i]``);
+    queries go to ``q_out`` (head j at columns j * head size of the cache, zeros behind its own
+    channels), keys and values into the paged cache at each token's position."""
+    _launch(_module("rotary"), "bt_head_rotary_call",
+            HeadRotaryCall(dtype=DTYPE_CODES[dtype], tokens=fused.shape[0], heads=heads, kv_heads=kv_heads, dim=dim,
+                           vdim=vdim, rot_dims=rot_dims, eps=eps, input=fused.data_ptr(), ld=fused.stride(0),
+                           q_gamma=_ptr(q_gamma), k_gamma=_ptr(k_gamma), inv_freq=_ptr(inv_freq),
+                           q_out=q_out.data_ptr(), ld_q=q_out.stride(0), tok_seq=tok_seq.data_ptr(),
+                           tok_pos=tok_pos.data_ptr(), kv=kv_view))
+
+
+# --- routed feed-forward ----------------------------------------------------------------------
+
+def route(h, router, correction, top, groups, keep, weights, gate_weight=None, gate=None):
+    """Per row of ``h``: softmax of the float32 router's logits over all experts, the ``top`` experts
+    with the largest score + ``correction`` among the best ``keep`` of ``groups`` equal groups (groups
+    <= 1: among all), and into ``weights`` [rows, experts] the chosen experts' scores divided by their
+    sum, zero elsewhere.  With ``gate_weight`` [width]: ``gate`` [rows] = sigmoid(gate_weight . h)."""
+    _launch(_module("experts"), "bt_route_call",
+            RouteCall(dtype=DTYPE_CODES[h.dtype], tokens=h.shape[0], width=router.shape[1], experts=router.shape[0],
+                      top=top, groups=groups, keep=keep, h=h.data_ptr(), ldh=h.stride(0), W=router.data_ptr(),
+                      correction=_ptr(correction), gate_w=_ptr(gate_weight), weights=weights.data_ptr(), gate=_ptr(gate)))
+
+
+def gated_experts(gu, weights, gate, experts, ff, shared_ff, identity, hidden, h=None, identity_out=None):
+    """hidden[t, e * ff + i] = weights[t, e] * silu(gate_e,i) * up_e,i from the rows ``gu`` of a fused
+    gate/up projection (per expert its gate rows, then its up rows; behind the experts the one every
+    token uses, weighted by ``gate[t]``); columns behind them are set to zero.  ``identity_out`` (float32
+    [rows, width]) receives (the sum of the identity experts' weights) * h."""
+    _launch(_module("experts"), "bt_gated_experts_call",
+            GatedExpertsCall(dtype=DTYPE_CODES[gu.dtype], tokens=gu.shape[0], experts=experts, ff=ff, shared_ff=shared_ff,
+                             identity=identity, hidden_cols=hidden.shape[1], width=h.shape[1] if h is not None else 0,
+                             gu=gu.data_ptr(), ld_gu=gu.stride(0), weights=weights.data_ptr(), gate=_ptr(gate),
+                             hidden=hidden.data_ptr(), ld_hidden=hidden.stride(0), h=_ptr(h),
+                             ldh=h.stride(0) if h is not None else 0, identity_out=_ptr(identity_out)))

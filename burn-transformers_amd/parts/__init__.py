@@ -1,8 +1,8 @@
-from . import (attention, block, feed_forward, latent_attention, norm, position, readout,  # noqa: F401  (registers the parts)
-               state_space)
+from . import (attention, block, experts, feed_forward, latent_attention, norm, position, readout,  # noqa: F401  (registers the parts)
+               reentry, rotary_attention, state_space)
 from .base import (Block, Delta, Embedding, FeedForward, Memory, Mixer, Norm, Part, Readout,
-                   ResidualStream)
+                   ResidualStream, Transform)
 from .registry import lookup, register, unregister
 
 __all__ = ["Block", "Delta", "Embedding", "FeedForward", "Memory", "Mixer", "Norm", "Part",
-           "Readout", "ResidualStream", "lookup", "register", "unregister"]
+           "Readout", "ResidualStream", "Transform", "lookup", "register", "unregister"]

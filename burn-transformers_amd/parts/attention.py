@@ -1,7 +1,8 @@
 """Causal self-attention with grouped heads over the paged cache.
 
 Parameters (all from the plan): width, heads, kv_heads, head_dim, scale (multiplies q.k),
-window (0 = every earlier key), causal.  Tensors: a fused projection ``qkv_weight`` held
+window (0 = every earlier key), chunk (0, or a query sees only the keys of its own chunk of that many
+positions, counted from position 0 of the sequence), causal.  Tensors: a fused projection ``qkv_weight`` held
 [heads*head_dim + 2*kv_heads*head_dim, width] with its bias, and ``out_weight`` [width,
 heads*head_dim] with its bias.
 
@@ -49,6 +50,7 @@ class CausalSelfAttention(Mixer):
         p = params
         self.width, self.heads, self.kv_heads = p["width"], p["heads"], p["kv_heads"]
         self.head_dim, self.scale, self.window = p["head_dim"], float(p["scale"]), int(p.get("window") or 0)
+        self.chunk = int(p.get("chunk") or 0)
         if not p.get("causal", True):
             raise ValueError("attention: only causal attention runs from a cache")
         if self.head_dim <= 0:
@@ -84,7 +86,7 @@ class CausalSelfAttention(Mixer):
         self.out_packed = packed_for_stream(self.out_weight) if self.out_weight.is_cuda else None
 
     def kv_spec(self):
-        return KVSpec(self.kv_heads, self.head_dim, self.window)
+        return KVSpec(self.kv_heads, self.head_dim, self.window, self.chunk)
 
     def kernel_modules(self, dtype):
         if self.plain_only:
@@ -98,7 +100,10 @@ class CausalSelfAttention(Mixer):
         context, not its exact lengths, so that every step of a class runs the same kernels."""
         if not step.decode:
             return 1
-        keys = min(step.context_limit, self.window + 32) if self.window else step.context_limit
+        keys = step.context_limit
+        for reach in (self.window, self.chunk):           # the most keys a query sees, a tile's slack added
+            if reach:
+                keys = min(keys, reach + 32)
         pair_bytes = keys * self.head_dim * 2 * (2 if step.dtype_is_bf16 else 4)     # one head's keys and values
         if pair_bytes <= SPLIT_BYTES:
             return 1
@@ -115,7 +120,7 @@ class CausalSelfAttention(Mixer):
         1,024 tokens 16.6 / 16.9 / 17.3 / 18.0, 2,048: 25.9 / 21.9 / 20.4 / 20.8, 4,096: 45.7 / 31.9 /
         25.5 / 25.3, 8,192: 84.5 / 51.9 / 35.6 / 33.7; two sequences (100 work-groups) 4,096: 48.1 /
         36.9, 8,192: 88.4 / 57.7."""
-        if step.decode or not step.dtype_is_bf16 or self.head_dim != 64 or self.window or self.plain_only:
+        if step.decode or not step.dtype_is_bf16 or self.head_dim != 64 or self.window or self.chunk or self.plain_only:
             return 1
         if step.context_limit <= PROMPT_RUN_MIN_CONTEXT:
             return 1
@@ -157,6 +162,6 @@ class CausalSelfAttention(Mixer):
             partial = step.buffer("attention.partial", tokens * self.heads * prompt_runs, self.head_dim + 2, "float32")
         args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
                                 self.heads, step.n_seqs, step.max_count, self.scale, self.window, partial,
-                                runs=prompt_runs if prompt_runs > 1 else None)
+                                runs=prompt_runs if prompt_runs > 1 else None, chunk=self.chunk)
         K.attention(args, step.dtype, step.decode, impl="plain" if self.plain_only else "auto")
         stream.add_product(step, mixed, self.out_weight, self.out_bias, packed=self.out_packed)

@@ -6,6 +6,7 @@
   FeedForward  forward(h, step) -> Delta
   Embedding    embed(step) -> ResidualStream             (token table and position encoding)
   Readout      logits(h, step) -> float32 [rows, vocab]
+  Transform    forward(stream, step)                     (replaces the stream's rows: a projection between runs of layers)
   Block        forward(stream, step, memory)             (the arrangement of the parts above)
 
 No part knows which model it is in: it gets its sizes and constants as parameters and its
@@ -46,6 +47,9 @@ class ResidualStream:
         # together with x; None where nobody keeps one.  Parts that read the stream itself, not a
         # norm of it, multiply by this (``operand``).
         self.cast = None
+        # the embedding's output, float32 [tokens, width], where the embedding keeps it for parts
+        # that read it again later (``keep_origin``); None otherwise
+        self.origin = None
 
     def operand(self, step):
         """The stream's rows as a product's operand: x itself in float32 models, its copy in the
@@ -232,6 +236,14 @@ class Readout(Part):
     takes_deferred_norm = False
 
     def logits(self, h, step):
+        raise NotImplementedError
+
+
+class Transform(Part):
+    """A part that stands between layers and replaces the residual stream's rows (a projection of
+    the stream, alone or with the embedding's output beside it).  It keeps nothing in the cache."""
+
+    def forward(self, stream, step):
         raise NotImplementedError
 
 

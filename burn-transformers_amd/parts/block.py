@@ -7,9 +7,15 @@ returns it as a Delta, which stays pending until the next norm reads the stream.
 output_norm: y = x + m * norm(mixer(x)); z = y + m * norm(feed_forward(y)), the feed-forward
 optional.  The parts read the stream itself; what is normalised is what they add.  ``m`` is the
 block's parameter ``mult``.
+
+sandwich_norm: y = x + post(mixer(pre(x))); z = y + post'(feed_forward(pre'(y))), the feed-forward
+optional: a norm before AND behind every sublayer, four norms a layer with tensors of their own.
+
+transform: x = t(x), one part of role "transform" and nothing else: what stands between two runs of
+layers (it keeps nothing in the cache; its schedule entry names no cache entry).
 """
 
-from .base import Block, SublayerOutput, offers_chunked
+from .base import Block, SublayerOutput, Transform, offers_chunked
 from .registry import register
 
 # Most rows of a step whose first norm is folded too.  Measured at GPT-2 XL sizes, ms a decode step
@@ -93,3 +99,51 @@ class OutputNormBlock(Block):
         if "ff" in parts:
             delta = parts["ff"].forward(stream.operand(step), step, output)
             parts["ff_norm"].add_output(stream, step, delta if delta is not None else output.take(), self.mult)
+
+
+@register("block", "sandwich_norm")
+class SandwichNormBlock(Block):
+    """A norm before and a norm behind each sublayer: the sublayer reads a norm of the stream, and
+    its output is normalised again before it joins the stream.  The norms behind are of a kind with
+    ``add_output`` (layer_norm, rms_norm).  A layer without a feed-forward leaves ``ff`` and its two
+    norms out."""
+    ROLES = {"mixer_norm": "norm", "mixer": "mixer", "mixer_post": "norm",
+             "ff_norm": "norm", "ff": "feed_forward", "ff_post": "norm"}
+    OPTIONAL = ("ff_norm", "ff", "ff_post")
+    only_launches_kernels = True
+
+    def __init__(self, parts, params=None):
+        super().__init__(parts, params)
+        if len({name in parts for name in ("ff_norm", "ff", "ff_post")}) != 1:
+            raise ValueError("sandwich_norm block: a feed-forward and its two norms come together")
+        for name in ("mixer_post", "ff_post"):
+            if name in parts and not hasattr(parts[name], "add_output"):
+                raise ValueError(f"sandwich_norm block: {type(parts[name]).__name__} cannot normalise a sublayer's output")
+
+    def forward(self, stream, step, memory):
+        parts = self.parts
+        output = SublayerOutput()
+        mixer = parts["mixer"]
+        h = _apply(parts["mixer_norm"], stream, step, mixer.takes_deferred_norm)
+        delta = mixer.forward(h, step, memory, output)
+        parts["mixer_post"].add_output(stream, step, delta if delta is not None else output.take(), keep_operand=False)
+        if "ff" in parts:
+            ff = parts["ff"]
+            h = _apply(parts["ff_norm"], stream, step, ff.takes_deferred_norm)
+            delta = ff.forward(h, step, output)
+            parts["ff_post"].add_output(stream, step, delta if delta is not None else output.take(), keep_operand=False)
+
+
+@register("block", "transform")
+class TransformBlock(Block):
+    """One part that replaces the stream's rows; no mixer, nothing in the cache."""
+    ROLES = {"transform": "transform"}
+    only_launches_kernels = True
+
+    def __init__(self, parts, params=None):
+        super().__init__(parts, params)
+        if not isinstance(parts["transform"], Transform):
+            raise ValueError(f"transform block: {type(parts['transform']).__name__} is no transform")
+
+    def forward(self, stream, step, memory):
+        self.parts["transform"].forward(stream, step)

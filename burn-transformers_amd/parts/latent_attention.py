@@ -96,6 +96,7 @@ class LatentAttention(Mixer):
     # the planning of a prompt's runs of keys is the ordinary attention's: one cached head, ``heads`` query heads
     kv_heads = 1
     window = 0
+    chunk = 0
     prompt_runs = CausalSelfAttention.prompt_runs
 
     def decode_runs(self, step, device):

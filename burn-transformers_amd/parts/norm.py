@@ -8,9 +8,13 @@ Parameter ``offset`` (default 0): the scale is stored as its distance from ``off
 multiplies by offset + weight (1 for scales stored around zero); the sum is formed once, in
 float32, when the part is built.
 
-``apply`` first adds what is pending on the residual stream, in the same pass.  ``add_output``
-(rms_norm) is the norm of a sublayer's OUTPUT: x += mult * norm(output), for layers that read the
-stream itself and normalise what they add to it.
+Parameter ``gain`` (default 1): scale and shift are multiplied by it once, in float32, when the part
+is built (a model that scales what it reads off the normalised rows, its logits for one, states
+the factor here).
+
+``apply`` first adds what is pending on the residual stream, in the same pass.  ``add_output`` is
+the norm of a sublayer's OUTPUT: x += mult * norm(output), for layers that normalise what they add
+to the stream (with or without a norm of the sublayer's input as well).
 """
 
 from ..kernels import library as K
@@ -31,6 +35,10 @@ class _KernelNorm(Norm):
         self.offset = float(params.get("offset", 0.0))
         if self.offset:
             self.weight = (self.weight.float() + self.offset).contiguous()
+        gain = float(params.get("gain", 1.0))
+        if gain != 1.0:
+            self.weight = (self.weight.float() * gain).contiguous()
+            self.bias = (self.bias.float() * gain).contiguous() if self.bias is not None else None
 
     def apply(self, stream, step, rows=None, chunked=False):
         count = rows.numel() if rows is not None else stream.x.shape[0]
@@ -55,6 +63,22 @@ class _KernelNorm(Norm):
         return K.Normalized(stream.x, self.weight, self.bias, self.eps, self.KIND)
 
 
+    def add_output(self, stream, step, delta, mult=1.0, accumulate=True, keep_operand=True):
+        """x (+)= mult * norm(v), v = the sublayer's output ``delta`` (a ``Delta``; None: the stream's
+        own rows, normalised in place).  In a bfloat16 model the new rows are also left as the
+        stream's copy in the products' type (``stream.operand``) unless ``keep_operand`` is False
+        (layers whose sublayers read a norm of the stream have no use for it)."""
+        if stream.pending is not None:
+            stream.flush()
+        cast = None
+        if keep_operand and step.dtype != stream.x.dtype:
+            cast = step.buffer("stream.operand", stream.x.shape[0], operand_columns(self.width, step.dtype), step.dtype)
+        K.output_norm(stream.x, self.weight, self.eps, mult, delta=delta.partials if delta is not None else None,
+                      bias=delta.bias if delta is not None else None, accumulate=accumulate, cast=cast,
+                      kind=self.KIND, beta=self.bias)
+        stream.cast = cast
+
+
 @register("norm", "layer_norm")
 class LayerNorm(_KernelNorm):
     KIND = "layer_norm"
@@ -63,16 +87,3 @@ class LayerNorm(_KernelNorm):
 @register("norm", "rms_norm")
 class RMSNorm(_KernelNorm):
     KIND = "rms_norm"
-
-    def add_output(self, stream, step, delta, mult=1.0, accumulate=True):
-        """x (+)= mult * v / sqrt(mean(v^2) + eps) * scale, v = the sublayer's output ``delta`` (a
-        ``Delta``; None: the stream's own rows, normalised in place).  In a bfloat16 model the new
-        rows are also left as the stream's copy in the products' type (``stream.operand``)."""
-        if stream.pending is not None:
-            stream.flush()
-        cast = None
-        if step.dtype != stream.x.dtype:
-            cast = step.buffer("stream.operand", stream.x.shape[0], operand_columns(self.width, step.dtype), step.dtype)
-        K.output_norm(stream.x, self.weight, self.eps, mult, delta=delta.partials if delta is not None else None,
-                      bias=delta.bias if delta is not None else None, accumulate=accumulate, cast=cast)
-        stream.cast = cast

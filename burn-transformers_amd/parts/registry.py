@@ -4,9 +4,9 @@ Adding a part means writing a class with the interface of ``parts/base.py`` and 
 under a new kind; plans may then name it layer by layer.
 """
 
-MIXERS, FEED_FORWARDS, NORMS, EMBEDDINGS, READOUTS, BLOCKS = {}, {}, {}, {}, {}, {}
+MIXERS, FEED_FORWARDS, NORMS, EMBEDDINGS, READOUTS, BLOCKS, TRANSFORMS = {}, {}, {}, {}, {}, {}, {}
 _TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "embedding": EMBEDDINGS,
-           "readout": READOUTS, "block": BLOCKS}
+           "readout": READOUTS, "block": BLOCKS, "transform": TRANSFORMS}
 
 
 def register(role, kind, cls=None, replace=False):

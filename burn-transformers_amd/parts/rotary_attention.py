@@ -1,0 +1,122 @@
+"""Causal self-attention whose queries and keys are normalised per head and turned by their
+positions (rotary positions), with grouped heads over the paged cache.
+
+Parameters (all from the plan): width, heads, kv_heads, dim (a query's and a key's head size), vdim
+(a value's head size, which may differ), scale (multiplies q.k), eps (of the head norms), head_norm
+(whether queries and keys are divided by their root mean square per head, times the scales
+``q_norm`` / ``k_norm`` [dim] that all heads share), rot_dims (the first so many channels of every
+query and key head are turned, channel i with channel i + rot_dims / 2, by the angle position *
+f_i), rot_base (f_i = rot_base^(-2 i / rot_dims)), rot_scaling (None, or factor / low / high /
+original: frequencies whose wavelength is beyond original / low are divided by factor, those whose
+wavelength is below original / high are kept, and between the two the division is blended in
+linearly in original / wavelength), window and chunk (which earlier keys a query sees, as in
+``parts/attention.py``).  Tensors: q_weight [heads * dim, width], k_weight [kv_heads * dim, width],
+v_weight [kv_heads * vdim, width], out_weight [width, heads * vdim], no biases.
+
+One step: ONE product with the three projections laid one behind the other leaves 32-bit sums; a
+kernel normalises and turns the heads, writes the queries to a buffer and the keys (turned) and
+values straight into the cache at each token's position; the framework's attention kernels read the
+cache; the output projection adds to the stream.  The cache keeps heads of one size, max(dim, vdim)
+rounded up to what the kernels take, with zeros behind a head's own channels; the output
+projection's columns are spread the same way, so the zeros meet zeros.
+"""
+
+import math
+
+import torch
+
+from ..kernels import library as K
+from .attention import CausalSelfAttention
+from .base import Mixer, packed_for_stream
+from .registry import register
+
+
+def rotary_frequencies(dims, base, scaling=None):
+    """f_i for i < dims / 2 (float64): base^(-2 i / dims), rescaled by ``scaling`` as the module's text says."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    if scaling:
+        factor, low, high, original = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+        wavelength = 2.0 * math.pi / f
+        blend = (original / wavelength - low) / (high - low)
+        between = (1.0 - blend) * f / factor + blend * f
+        f = torch.where(wavelength < original / high, f, torch.where(wavelength > original / low, f / factor, between))
+    return f
+
+
+@register("mixer", "rotary_attention")
+class RotaryAttention(CausalSelfAttention):
+    takes_deferred_norm = False          # (its first product leaves 32-bit sums; the rows come normalised)
+    only_launches_kernels = True
+
+    def __init__(self, params, tensors):
+        Mixer.__init__(self, params, tensors)
+        p = params
+        self.width, self.heads, self.kv_heads = p["width"], p["heads"], p["kv_heads"]
+        self.dim, self.vdim = p["dim"], p["vdim"]
+        self.scale, self.eps = float(p["scale"]), float(p.get("eps", 0.0))
+        self.window, self.chunk = int(p.get("window") or 0), int(p.get("chunk") or 0)
+        self.rot_dims = int(p.get("rot_dims") or 0)
+        if self.heads % self.kv_heads != 0:
+            raise ValueError(f"rotary attention: {self.heads} query heads cannot share {self.kv_heads} key/value heads")
+        if self.rot_dims % 2 != 0 or self.rot_dims > self.dim:
+            raise ValueError(f"rotary attention: {self.rot_dims} turned channels must be even and at most the head size {self.dim}")
+        shapes = {"q_weight": (self.heads * self.dim, self.width), "k_weight": (self.kv_heads * self.dim, self.width),
+                  "v_weight": (self.kv_heads * self.vdim, self.width), "out_weight": (self.width, self.heads * self.vdim)}
+        if p.get("head_norm", True):
+            shapes.update(q_norm=(self.dim,), k_norm=(self.dim,))
+        for role, shape in shapes.items():
+            if tuple(tensors[role].shape) != shape:
+                raise ValueError(f"rotary attention: {role} is {tuple(tensors[role].shape)}, expected {shape}")
+        self.q_norm, self.k_norm = tensors.get("q_norm"), tensors.get("k_norm")
+        dtype = tensors["q_weight"].dtype
+        bf16 = dtype == torch.bfloat16
+        # the cached head: the larger of the two head sizes, in the steps of 16 the MFMA kernels take
+        self.head_dim = (max(self.dim, self.vdim) + 15) // 16 * 16
+        if self.head_dim > 256:
+            raise ValueError(f"rotary attention: heads of {max(self.dim, self.vdim)} are beyond 256, the most any kernel here takes")
+        if bf16 and self.head_dim > 128:
+            raise ValueError(f"rotary attention: the bfloat16 kernels take heads of up to 128, not {self.head_dim}; "
+                             f"load the model with dtype float32")
+        self.plain_only = False
+        self.n_q, self.n_kv = self.heads * self.head_dim, self.kv_heads * self.head_dim
+        self.fused_cols = (self.heads + self.kv_heads) * self.dim + self.kv_heads * self.vdim
+        self.qkv_weight = torch.cat([tensors["q_weight"], tensors["k_weight"], tensors["v_weight"]]).contiguous()
+        # the output projection reads heads of head_dim: its columns are spread, zeros between them
+        out = tensors["out_weight"]
+        spread = out.new_zeros(self.width, self.heads, self.head_dim)
+        spread[:, :, :self.vdim] = out.view(self.width, self.heads, self.vdim)
+        self.out_weight = spread.view(self.width, self.n_q).contiguous()
+        self.out_bias = None
+        device = self.qkv_weight.device
+        self.inv_freq = rotary_frequencies(self.rot_dims, p["rot_base"], p.get("rot_scaling")).to(torch.float32).to(device) \
+            if self.rot_dims else None
+        on_gpu = self.qkv_weight.is_cuda
+        self.qkv_packed = K.PackedWeight(self.qkv_weight) if on_gpu else None
+        self.out_packed = packed_for_stream(self.out_weight) if on_gpu else None
+
+    def kernel_modules(self, dtype):
+        return ("rotary",) + tuple(super().kernel_modules(dtype))
+
+    def forward(self, h, step, memory, stream):
+        tokens = h.shape[0]
+        if not memory.writes:
+            raise ValueError("rotary attention: every run keeps a cache entry of its own")
+        kv = memory.kv()
+        fused = step.buffer("rotary.fused", tokens, self.fused_cols, "float32")
+        K.gemm(h, self.qkv_weight, K.epilogue_f32(fused), packed=self.qkv_packed)
+        q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
+        K.head_rotary(fused, self.heads, self.kv_heads, self.dim, self.vdim, self.rot_dims, self.inv_freq,
+                      self.q_norm, self.k_norm, self.eps, q, step.tok_seq, step.tok_pos, kv, step.dtype)
+        if step.decode and step.dtype_is_bf16 and K.Chunked.wanted(tokens) and self.heads // self.kv_heads <= 16:
+            mixed = K.Chunked.take(step, "attention.mixed", tokens, self.n_q, step.dtype)
+        else:
+            mixed = step.buffer("attention.mixed", tokens, self.n_q, step.dtype)
+        partial, runs = None, self.decode_runs(step, h.device)
+        if runs > 1:
+            partial = step.buffer("attention.partial", step.n_seqs * self.heads * runs, self.head_dim + 2, "float32")
+        args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
+                                self.heads, step.n_seqs, step.max_count, self.scale, self.window, partial,
+                                chunk=self.chunk)
+        K.attention(args, step.dtype, step.decode)
+        stream.add_product(step, mixed, self.out_weight, None, packed=self.out_packed)
