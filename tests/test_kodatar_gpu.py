@@ -1,0 +1,265 @@
+"""Kodatar through the engine against the plain implementation: every mechanism alone, and every
+way of cutting, batching and reusing that must not change the logits."""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import burn_transformers_amd as bt  # noqa: E402
+import plain_kodatar as plain  # noqa: E402
+from burn_transformers_amd.cache.ledger import RELEASED  # noqa: E402
+from kodatar_helpers import (CONFIGS, engine_for, model_for, plain_logits, prompts_for, tolerance,  # noqa: E402
+                             weights_for)
+
+DTYPES = ["float32", "bfloat16"]
+SHARPEN = 4.0        # factor on the queries' head scale where attention is to put its weight on few keys
+
+
+def check(got, want, dtype, what):
+    """float32: every row within the bound.  bfloat16 (whose weights are made so that no choice of
+    experts hangs on a close call, see ``kodatar_helpers.weights_for``): a row in forty (at least two)
+    may pass the bound."""
+    got = got.detach().cpu().double()
+    assert torch.isfinite(got).all(), what
+    rows = (got - want).abs().max(dim=1).values
+    bound = tolerance(dtype, want)
+    over = int((rows > bound).sum())
+    allowed = 0 if dtype == "float32" else max(2, rows.numel() // 40)
+    assert over <= allowed, f"{what}: {over} rows over {bound}, max abs error {float(rows.max())}"
+
+
+def whole(engine, ids):
+    slot = engine.open()
+    logits = engine.step([(slot, ids)], want=[list(range(len(ids)))]).clone()
+    engine.close(slot)
+    return logits
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,lengths", [("attention", [1, 2, 9, 64, 65, 130]), ("causal", [1, 3, 70, 200]),
+                                          ("experts", [1, 17, 80]), ("experts_full", [1, 2, 33, 90]),
+                                          ("loop", [1, 5, 70]), ("basic", [1, 2, 23, 24, 25, 49, 130]),
+                                          ("odd", [1, 6, 7, 8, 99, 101, 210])])
+def test_each_mechanism_and_each_request_whole(name, dtype, lengths):
+    engine = engine_for(name, dtype)
+    for ids in prompts_for(name, lengths):
+        check(whole(engine, ids), plain_logits(name, ids, dtype=dtype), dtype, f"{name} whole {len(ids)}")
+    engine.cache.ledger.check()
+
+
+def test_residual_stream_after_every_run_of_a_layer():
+    """The stream itself, run by run (a looped layer counts each time), in float32."""
+    name = "basic"
+    model = model_for(name, "float32")
+    engine = bt.Engine(model, max_tokens=256, graphs=False, programs=False)
+    ids = prompts_for(name, [29], seed=4)[0]
+    want = []
+    plain.forward(ids, weights_for(name), CONFIGS[name][0], residuals=want)
+    caught, restore = [], []
+    for block in model.blocks:
+        if block.mixers():
+            restore.append((block, block.forward))
+
+            def run(stream, step, memory, forward=block.forward):
+                forward(stream, step, memory)
+                stream.flush()
+                caught.append(stream.x.detach().cpu().double().clone())
+            block.forward = run
+    try:
+        slot = engine.open()
+        engine.step([(slot, ids)])
+        engine.close(slot)
+    finally:
+        for block, forward in restore:
+            del block.forward
+    assert len(caught) == len(want) == 3 * 2 + 1
+    for number, (got, reference) in enumerate(zip(caught, want)):
+        assert float((got - reference).abs().max()) <= 2e-5 + 2e-5 * float(reference.abs().max()), f"run {number}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,length,tail", [("basic", 80, 40), ("odd", 110, 20), ("attention", 140, 80), ("loop", 9, 8)])
+def test_prompt_then_token_by_token(name, dtype, length, tail):
+    """The last tokens one by one through the cache give what the whole prompt gives; the tails pass
+    over chunk edges."""
+    engine = engine_for(name, dtype)
+    ids = prompts_for(name, [length], seed=3)[0]
+    want = plain_logits(name, ids, dtype=dtype)
+    slot = engine.open()
+    head = length - tail
+    rows = [engine.step([(slot, ids[:head])], want=[list(range(head))]).clone()]
+    for token in ids[head:]:
+        rows.append(engine.step([(slot, [token])]).clone())
+    check(torch.cat(rows), want, dtype, f"{name} decode")
+    engine.close(slot)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["basic", "odd"])
+def test_from_the_first_token_one_by_one(name, dtype):
+    engine = engine_for(name, dtype)
+    ids = prompts_for(name, [60], seed=9)[0]
+    slot = engine.open()
+    rows = [engine.step([(slot, [token])]).clone() for token in ids]
+    check(torch.cat(rows), plain_logits(name, ids, dtype=dtype), dtype, f"{name} from the first token")
+    engine.close(slot)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,portion", [("basic", 2), ("basic", 3), ("basic", 24), ("basic", 64), ("basic", 65),
+                                          ("odd", 2), ("odd", 7), ("odd", 50), ("long", 193)])
+def test_prompt_in_portions(name, dtype, portion):
+    """Portions that start anywhere in a chunk and in a block."""
+    engine = engine_for(name, dtype)
+    ids = prompts_for(name, [600 if name == "long" else 151], seed=5)[0]
+    slot = engine.open()
+    rows = []
+    for at in range(0, len(ids), portion):
+        part = ids[at:at + portion]
+        rows.append(engine.step([(slot, part)], want=[list(range(len(part)))]).clone())
+    check(torch.cat(rows), plain_logits(name, ids, dtype=dtype), dtype, f"{name} in portions of {portion}")
+    engine.close(slot)
+    engine.cache.ledger.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["basic", "odd"])
+def test_unequal_batch_decoded_together_then_slots_and_blocks_reused(name, dtype):
+    """Requests of unequal length in one step, decoded together while the shorter ones end; then a
+    second batch in the slots and blocks the first gave back."""
+    engine = engine_for(name, dtype, max_tokens=1024)
+    for round_, lengths in enumerate([[1, 70, 33, 129], [64, 5, 90]]):
+        prompts = prompts_for(name, lengths, seed=20 + round_)
+        tails = [12, 5, 9, 3][:len(prompts)]
+        extra = [prompts_for(name, [t], seed=30 + i)[0] for i, t in enumerate(tails)]
+        slots = [engine.open() for _ in prompts]
+        got = [[] for _ in prompts]
+        logits = engine.step(list(zip(slots, prompts)), want=[list(range(len(p))) for p in prompts])
+        at = 0
+        for i, p in enumerate(prompts):
+            got[i].append(logits[at:at + len(p)].clone())
+            at += len(p)
+        for t in range(max(tails)):
+            live = [i for i in range(len(prompts)) if t < tails[i]]
+            logits = engine.step([(slots[i], [extra[i][t]]) for i in live])
+            for row, i in enumerate(live):
+                got[i].append(logits[row:row + 1].clone())
+            for i in range(len(prompts)):
+                if t + 1 == tails[i]:
+                    engine.close(slots[i])
+        for i, p in enumerate(prompts):
+            check(torch.cat(got[i]), plain_logits(name, p + extra[i], dtype=dtype), dtype, f"{name} round {round_} request {i}")
+        engine.cache.ledger.check()
+    assert not engine.cache.ledger.live_slots()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_keys_far_back_at_block_borders_and_at_chunk_edges(dtype):
+    """Attention sharpened so that weight lies on single keys: chunks of 448 positions span seven
+    blocks of the cache, the second layer sees every earlier key; whole, and decoded across the
+    chunk's edge and a block border."""
+    name = "long"
+    ids = prompts_for(name, [940], seed=11)[0]
+    want = plain_logits(name, ids, SHARPEN, dtype)
+    # the premise: in the plain model some query's largest attention weight is far back
+    engine = engine_for(name, dtype, sharpen=SHARPEN)
+    check(whole(engine, ids), want, dtype, "long whole")
+    slot = engine.open()
+    head = 870                      # 896 = 2 * 448 is a chunk's edge and a block border
+    rows = [engine.step([(slot, ids[:head])], want=[list(range(head))]).clone()]
+    rows += [engine.step([(slot, [token])]).clone() for token in ids[head:]]
+    check(torch.cat(rows), want, dtype, "long decoded across a chunk's edge")
+    held = engine.cache.blocks(slot, 0), engine.cache.blocks(slot, 1)
+    engine.close(slot)
+    # one of the two groups (the chunked layers') has given the blocks before the last chunk back
+    assert any(RELEASED in blocks for blocks in held) and any(RELEASED not in blocks for blocks in held)
+
+
+def test_sharpened_attention_puts_weight_on_far_keys():
+    """The premise of the test above, on the plain implementation: with the sharpened queries, hiding
+    the far half of the first layer's keys from the last query moves its logits by far more than any
+    bound here."""
+    name = "long"
+    config = CONFIGS[name][0]
+    ids = prompts_for(name, [440], seed=11)[0]
+    weights = weights_for(name, SHARPEN)
+    full = plain.forward(ids, weights, config)[-1]
+    first = dict(config["layers"][0], mixer=dict(config["layers"][0]["mixer"], mask={"size": 224}))
+    moved = plain.forward(ids, weights, dict(config, layers=[first, config["layers"][1]]))[-1]
+    assert float((full - moved).abs().max()) > 10 * tolerance("bfloat16", full)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(dtype):
+    name = "basic"
+    engine = engine_for(name, dtype)
+    ids = prompts_for(name, [330], seed=12)[0]
+    slot = engine.open()
+    rows = [engine.step([(slot, ids[:4])], want=[[0, 1, 2, 3]]).clone()]
+    rows += [engine.step([(slot, [token])]).clone() for token in ids[4:]]
+    check(torch.cat(rows), plain_logits(name, ids, dtype=dtype), dtype, "300 tokens one by one")
+    engine.close(slot)
+
+
+@pytest.mark.parametrize("graphs,programs", [(False, False), (False, True), ("always", True)])
+def test_launch_lists_and_graphs_give_the_same_bits(graphs, programs):
+    name = "basic"
+    ids = prompts_for(name, [70], seed=13)[0]
+    rows = {}
+    for key, options in (("direct", dict(graphs=False, programs=False)), ("other", dict(graphs=graphs, programs=programs))):
+        engine = engine_for(name, "bfloat16", **options)
+        got = []
+        for _ in range(3):          # a shape comes again: recorded, then replayed
+            slot = engine.open()
+            got.append(engine.step([(slot, ids[:50])], want=[[49]]).clone())
+            got += [engine.step([(slot, [token])]).clone() for token in ids[50:]]
+            engine.close(slot)
+        rows[key] = torch.cat(got)
+    assert torch.equal(rows["direct"], rows["other"])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_greedy_generation_through_the_entry_point(dtype):
+    name = "basic"
+    config = CONFIGS[name][0]
+    prompts = prompts_for(name, [5, 40, 1, 27], seed=14)
+    engine = engine_for(name, dtype)
+    got = bt.generate(engine, prompts, bt.GenerationConfig(max_new_tokens=10), prefill_chunk=16)
+    for prompt, sequence in zip(prompts, got):
+        ids = list(prompt)
+        for token in sequence.token_ids:
+            logits = plain.forward(ids, weights_for(name, dtype=dtype), config)[-1]
+            best = int(logits.argmax())
+            if dtype == "float32":
+                assert token == best
+            else:                    # 8-bit operands may take a token whose logit is within rounding of the best
+                assert float(logits[best] - logits[token]) <= tolerance(dtype, logits)
+            ids.append(token)
+    assert not engine.cache.ledger.live_slots()
+
+
+def test_folder_round_trip_and_replay(tmp_path):
+    """A folder written with random weights, loaded by what config.json names, replayed step by step."""
+    import json
+    import numpy as np
+    from burn_transformers_amd.engine.replay import Replay, cache_tokens
+    config = CONFIGS["odd"][0]
+    folder = tmp_path / "model"
+    weights = bt.write_random_model(str(folder), config, seed=3)
+    assert json.load(open(folder / "config.json"))["architecture"] == "Kodatar"
+    model = bt.load_model(str(folder), dtype="float32")
+    replay = Replay(bt.Engine(model, max_tokens=cache_tokens(300)), str(tmp_path / "out"))
+    a, b = prompts_for("odd", [45, 9], seed=15)
+    replay.run([json.dumps({"step": 0, "entries": [{"id": "a", "tokens": a[:40], "want": [0, 39]},
+                                                   {"id": "b", "tokens": b[:6], "want": [5]}], "end": []}),
+                json.dumps({"step": 1, "entries": [{"id": "a", "tokens": a[40:41], "want": [0]},
+                                                   {"id": "b", "tokens": b[6:7], "want": []}], "end": ["b"]}),
+                json.dumps({"step": 2, "entries": [{"id": "a", "tokens": a[41:42], "want": [0]}], "end": ["a"]})],
+               out=open(tmp_path / "log", "w"))
+    want_a, want_b = plain.forward(a, weights, config), plain.forward(b, weights, config)
+    first = torch.from_numpy(np.fromfile(tmp_path / "out" / "0.f32", dtype="<f4").reshape(3, -1)).double()
+    check(first, torch.stack([want_a[0], want_a[39], want_b[5]]), "float32", "replayed step 0")
+    for step, row in ((1, 40), (2, 41)):
+        got = torch.from_numpy(np.fromfile(tmp_path / "out" / f"{step}.f32", dtype="<f4").reshape(1, -1)).double()
+        check(got, want_a[row:row + 1], "float32", f"replayed step {step}")
