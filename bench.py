@@ -1,7 +1,7 @@
 """Throughput of GPT-2 generation on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers 48] [--dtype bf16]
-                    [--repetitions 10] [--workload xl|small|medium|sweep|salopel] [--model xl|medium|small]
+                    [--repetitions 10] [--workload xl|small|medium|sweep|salopel|kodatar] [--model xl|medium|small]
                     [--kernel-batches 1,64] [--sweep-part all|decode|prompts] [--no-points] [--no-kernels] [--no-own]
 
 The default workload (``xl``) has the layer sizes of GPT-2 XL with random weights: a batch of 8
@@ -47,6 +47,8 @@ and sampled at temperature 1 to 1,024 tokens each.  Their value is generated tok
 ``--workload salopel`` runs the library's second family, Salopel, at two widths whose layers resemble
 a real model's, beside GPT-2 at equal width, depth, feed-forward and vocabulary: prompt and decode
 throughput and each model's classes of kernels, one JSON line per width.
+``--workload kodatar`` does the same for the third family, Kodatar (rotary attention in chunks, routed
+experts, a stretch of layers that runs twice), beside GPT-2 at equal width, runs of layers and vocabulary.
 """
 
 import argparse
@@ -222,6 +224,17 @@ def _class_of(name, call):
         return f"head_scan {call.tokens}x{call.heads}x{call.vdim}x{call.state}", \
             call.n_seqs * inner * call.state * 8 + call.tokens * (inner * 8 + call.groups * call.state * 8), \
             6.0 * call.tokens * inner * call.state
+    if short == "head_rotary":
+        columns = (call.heads + call.kv_heads) * call.dim + call.kv_heads * call.vdim
+        return f"head_rotary {call.tokens}tok", call.tokens * columns * 6, 0.0
+    if short == "route":
+        return f"route {call.tokens}x{call.experts}", call.experts * call.width * 4 + call.tokens * call.width * 2, \
+            2.0 * call.tokens * call.experts * call.width
+    if short == "gated_experts":
+        element = 4 if call.dtype == 0 else 2
+        return f"gated_experts {call.tokens}x{call.hidden_cols}", call.tokens * call.hidden_cols * 3 * element, 0.0
+    if short == "join_rows":
+        return f"join_rows {call.tokens}x{call.width}", call.tokens * call.width * (8 + 2 * (4 if call.out_dtype == 0 else 2)), 0.0
     if short == "gated_norm":
         return f"gated_norm {call.tokens}x{call.channels}", call.tokens * call.channels * 10, 0.0
     return short, 0, 0.0
@@ -527,6 +540,7 @@ def salopel_config(width, layers, vocab):
 
 
 def build_salopel(config, dtype):
+    """A model of any family with the random weights its own initialisation draws."""
     import torch
 
     import burn_transformers_amd as bt
@@ -536,9 +550,41 @@ def build_salopel(config, dtype):
                                  dtype="bfloat16" if dtype == "bf16" else "float32")
 
 
+def kodatar_config(width, layers, vocab):
+    """Kodatar at layer sizes that resemble a real model's: ``layers`` runs of layers, of which the first
+    two thirds are one stretch of a third run twice; query heads of 128 on a quarter as many
+    key/value heads, values of 64, all of a head turned with rescaled frequencies, keys seen in chunks of
+    512; eight experts of the model's width of which a token uses two, one identity expert, in three
+    groups of which two stay open, and a shared expert of twice the width."""
+    heads = max(4, width // 128)
+    layer = {"type": "attention",
+             "mixer": {"heads": heads, "kv_heads": heads // 4, "dim": 128, "vdim": 64, "scale": 128 ** -0.5,
+                       "rot": {"dims": 128, "base": 500000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
+                       "mask": {"size": 512}},
+             "mlp": {"kind": "moe", "expert": {"ff": width},
+                     "router": {"experts": 8, "top": 2, "identity": 1, "groups": {"count": 3, "keep": 2}},
+                     "shared": {"ff": 2 * width}}}
+    third = max(1, layers // 3)
+    return {"architecture": "Kodatar", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "logit_scale": 1.0,
+            "norm": {"eps": 1e-5}, "loop": {"start": 0, "stop": third, "times": 2},
+            "layers": [dict(layer) for _ in range(layers - third)]}
+
+
 def run_salopel(args):
     """Prompt and decode throughput of Salopel beside GPT-2 at equal width, depth, feed-forward and
     vocabulary, with each model's classes of kernels on their own.  One JSON line per width."""
+    run_beside_gpt2(args, "salopel", salopel_config, lambda width: (2 * 128, 128 * min(16, width // 64)))
+
+
+def run_kodatar(args):
+    """The same for Kodatar: equal width, runs of layers and vocabulary."""
+    run_beside_gpt2(args, "kodatar", kodatar_config,
+                    lambda width: (2 * 128 * (max(4, width // 128) // 4), 128 * max(4, width // 128)))
+
+
+def run_beside_gpt2(args, family, config_of, attention_sizes):
+    """``attention_sizes(width)``: (cached values a token and layer, columns of a token's queries), for
+    the attention kernels' bytes and flops."""
     import torch
 
     import burn_transformers_amd as bt
@@ -546,11 +592,12 @@ def run_salopel(args):
     layers, batch, prompt_len, steps = args.layers or 12, args.batch, 512, min(args.steps, 64)
     vocab = 32000
     for width in (1024, 2048):
-        line = {"workload": "salopel beside gpt2", "width": width, "layers": layers, "dtype": dtype, "batch": batch,
+        cached, columns = attention_sizes(width)
+        line = {"workload": f"{family} beside gpt2", "width": width, "layers": layers, "dtype": dtype, "batch": batch,
                 "prompt_len": prompt_len, "decode_steps": steps, "data": "synthetic token ids, random weights"}
-        for name in ("salopel", "gpt2"):
-            if name == "salopel":
-                config = salopel_config(width, layers, vocab)
+        for name in (family, "gpt2"):
+            if name == family:
+                config = config_of(width, layers, vocab)
                 model = build_salopel(config, dtype)
             else:
                 config = dict(XL, n_layer=layers, n_embd=width, n_head=width // 64, n_inner=4 * width, vocab_size=vocab,
@@ -569,15 +616,15 @@ def run_salopel(args):
                 prompts = synthetic_prompts(batch, context - 1, vocab, seed=7)
                 slots = [engine.open() for _ in prompts]
                 engine.step(list(zip(slots, prompts)))
-                kv = batch * context * 2 * 128 * ELEMENT_BYTES[dtype] if name == "salopel" else batch * context * 2 * width * ELEMENT_BYTES[dtype]
-                flops = 4.0 * batch * context * (128 * min(16, width // 64) if name == "salopel" else width)
+                kv = batch * context * cached * ELEMENT_BYTES[dtype] if name == family else batch * context * 2 * width * ELEMENT_BYTES[dtype]
+                flops = 4.0 * batch * context * (columns if name == family else width)
                 result["decode_kernels"] = kernel_classes(engine, [(slot, [5]) for slot in slots], kv, flops, PEAK_FLOPS[dtype])
                 for slot in slots:
                     engine.close(slot)
                 prompts = synthetic_prompts(PREFILL_SEQS, PREFILL_LEN, vocab, seed=8)
                 slots = [engine.open() for _ in prompts]
                 tokens = PREFILL_SEQS * PREFILL_LEN
-                per_token = 128 * min(16, width // 64) if name == "salopel" else width
+                per_token = columns if name == family else width
                 result["prefill_kernels"] = kernel_classes(engine, list(zip(slots, prompts)), 4 * tokens * per_token * ELEMENT_BYTES[dtype],
                                                            PREFILL_SEQS * 2.0 * per_token * PREFILL_LEN * (PREFILL_LEN + 1),
                                                            PEAK_FLOPS[dtype], replays=10)
@@ -601,7 +648,7 @@ def main():
     parser.add_argument("--kernel-batches", default="", help="further batch sizes whose decode kernel classes are timed, e.g. 1,64")
     parser.add_argument("--dtype", choices=["bf16", "fp32"], default=None)
     parser.add_argument("--repetitions", type=int, default=10, help="measured repetitions, each on fresh sequences")
-    parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep", "salopel"], default="xl")
+    parser.add_argument("--workload", choices=["xl", "small", "medium", "sweep", "salopel", "kodatar"], default="xl")
     parser.add_argument("--sweep-part", choices=["all", "decode", "prompts"], default="all",
                         help="which table of --workload sweep to run")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
@@ -614,8 +661,8 @@ def main():
     if args.repetitions < 1:
         parser.error("--repetitions must be at least 1")
     args.kernel_batches = [int(b) for b in args.kernel_batches.split(",") if b]
-    if args.workload == "salopel":
-        run_salopel(args)
+    if args.workload in ("salopel", "kodatar"):
+        (run_salopel if args.workload == "salopel" else run_kodatar)(args)
         return
     if args.layers is None:
         args.layers = XL["n_layer"] if args.workload == "sweep" else MODELS[args.model]["n_layer"]

@@ -30,78 +30,118 @@ struct RouteCall {
   float* gate;              // [tokens]: sigmoid(gate_w . h), or null
 };
 
+#define ROUTE_BATCH 16          // router outputs whose sums a thread carries at once
+
+// The best (value, index) of a wave; among equal values the lowest index.  Every lane gets it.
+__device__ __forceinline__ void wave_best(float& value, int& index) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float other = __shfl_xor(value, o, 64);
+    const int other_index = __shfl_xor(index, o, 64);
+    if (other > value || (other == value && other_index < index)) { value = other; index = other_index; }
+  }
+}
+
+// One work-group per token.  Logits: a thread takes the columns t, t + 256, ... of the row and carries
+// the sums of ROUTE_BATCH outputs at once, so that all loads of a batch are in flight together (a
+// decode step has few tokens: one round trip to memory is the kernel's time); the sums meet through
+// wave reductions and LDS.  Everything after the logits is the first wave's alone, the experts dealt
+// to its lanes, maxima and choices as wave reductions: no barrier, no serial scan.
 template <typename T>
 __global__ void __launch_bounds__(ROUTE_THREADS) route_kernel(RouteCall c) {
-  extern __shared__ float hrow[];                 // [width]
+  __shared__ float partial[ROUTE_THREADS / 64][ROUTE_BATCH];
   __shared__ float score[ROUTE_MAX_EXPERTS];      // logits, then softmax scores
   __shared__ float choice[ROUTE_MAX_EXPERTS];     // scores with the correction; -inf once taken or shut out
-  __shared__ float scratch[32];
-  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = ROUTE_THREADS / 64;
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* h = static_cast<const T*>(c.h) + (int64_t)t * c.ldh;
-  for (int col = threadIdx.x; col < c.width; col += ROUTE_THREADS) hrow[col] = to_float(h[col]);
-  __syncthreads();
   const int outputs = c.experts + (c.gate_w ? 1 : 0);
-  for (int e = wave; e < outputs; e += waves) {
-    const float* w = e < c.experts ? c.W + (int64_t)e * c.width : c.gate_w;
-    float sum = 0.f;
-    for (int col = lane; col < c.width; col += 64) sum = fmaf(w[col], hrow[col], sum);
-    sum = wave_sum(sum);
-    if (lane == 0) {
+  for (int first = 0; first < outputs; first += ROUTE_BATCH) {
+    float sums[ROUTE_BATCH];
+#pragma unroll
+    for (int j = 0; j < ROUTE_BATCH; ++j) sums[j] = 0.f;
+    for (int col = threadIdx.x; col < c.width; col += ROUTE_THREADS) {
+      const float x = to_float(h[col]);
+#pragma unroll
+      for (int j = 0; j < ROUTE_BATCH; ++j) {
+        const int e = first + j;
+        if (e < outputs) sums[j] = fmaf((e < c.experts ? c.W + (int64_t)e * c.width : c.gate_w)[col], x, sums[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < ROUTE_BATCH; ++j) {
+      const float sum = wave_sum(sums[j]);
+      if (lane == 0) partial[wave][j] = sum;
+    }
+    __syncthreads();
+    if (threadIdx.x < ROUTE_BATCH && first + (int)threadIdx.x < outputs) {
+      float sum = 0.f;
+      for (int w = 0; w < ROUTE_THREADS / 64; ++w) sum += partial[w][threadIdx.x];
+      const int e = first + threadIdx.x;
       if (e < c.experts) score[e] = sum;
       else c.gate[t] = 1.0f / (1.0f + expf(-sum));
     }
+    __syncthreads();
   }
-  __syncthreads();
+  if (wave != 0) return;
   float top_logit = -INFINITY;
-  for (int e = threadIdx.x; e < c.experts; e += ROUTE_THREADS) top_logit = fmaxf(top_logit, score[e]);
-  top_logit = block_max(top_logit, scratch);
+  for (int e = lane; e < c.experts; e += 64) top_logit = fmaxf(top_logit, score[e]);
+  top_logit = wave_max(top_logit);
   float total = 0.f;
-  for (int e = threadIdx.x; e < c.experts; e += ROUTE_THREADS) total += expf(score[e] - top_logit);
-  total = block_sum(total, scratch);
-  __syncthreads();
-  for (int e = threadIdx.x; e < c.experts; e += ROUTE_THREADS) {
+  for (int e = lane; e < c.experts; e += 64) total += expf(score[e] - top_logit);
+  total = wave_sum(total);
+  float* weights = c.weights + (int64_t)t * c.experts;
+  for (int e = lane; e < c.experts; e += 64) {     // a lane keeps to its own experts: no other lane reads them yet
     const float s = expf(score[e] - top_logit) / total;
     score[e] = s;
     choice[e] = s + (c.correction ? c.correction[e] : 0.f);
-    c.weights[(int64_t)t * c.experts + e] = 0.f;
+    weights[e] = 0.f;
   }
-  __syncthreads();
-  if (threadIdx.x != 0) return;
-  // the choice itself is short and serial: a few hundred comparisons
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   if (c.groups > 1) {
     // a group's score is its best corrected score; the best `keep` groups stay open, the experts of
-    // the others are shut out (minus infinity, since corrected scores may be negative)
+    // the others are shut out (minus infinity, since corrected scores may be negative).  Lane g
+    // holds group g (at most 64 groups).
     const int per = c.experts / c.groups;
-    unsigned long long open = 0ull;
+    float group_score = -INFINITY;
+    if (lane < c.groups)
+      for (int i = 0; i < per; ++i) group_score = fmaxf(group_score, choice[lane * per + i]);
+    bool open = false;
     for (int kept = 0; kept < c.keep; ++kept) {
-      int best = -1;
-      float best_score = -INFINITY;
-      for (int g = 0; g < c.groups; ++g) {
-        if ((open >> g) & 1ull) continue;
-        float group_score = -INFINITY;
-        for (int i = 0; i < per; ++i) group_score = fmaxf(group_score, choice[g * per + i]);
-        if (best < 0 || group_score > best_score) { best = g; best_score = group_score; }
-      }
-      open |= 1ull << best;
+      float value = (lane < c.groups && !open) ? group_score : -INFINITY;
+      int index = (lane < c.groups && !open) ? lane : 0x7fffffff;
+      // (a group whose score is minus infinity itself still ranks before no group at all)
+      unsigned long long candidates = __builtin_amdgcn_ballot_w64(lane < c.groups && !open);
+      wave_best(value, index);
+      if (index == 0x7fffffff) index = __builtin_ctzll(candidates);
+      if (lane == index) open = true;
     }
-    for (int g = 0; g < c.groups; ++g)
-      if (!((open >> g) & 1ull))
-        for (int i = 0; i < per; ++i) choice[g * per + i] = -INFINITY;
+    if (lane < c.groups && !open)
+      for (int i = 0; i < per; ++i) choice[lane * per + i] = -INFINITY;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
   float sum = 0.f;
-  int chosen[64];
-  const int top = c.top < 64 ? c.top : 64;
-  for (int k = 0; k < top; ++k) {
-    int best = 0;
-    float best_score = choice[0];
-    for (int e = 1; e < c.experts; ++e)
-      if (choice[e] > best_score) { best = e; best_score = choice[e]; }
-    chosen[k] = best;
-    choice[best] = -INFINITY;
-    sum += score[best];
+  int mine = -1;                                   // lane k keeps the k-th chosen expert
+  for (int k = 0; k < c.top; ++k) {
+    float value = -INFINITY;
+    int index = 0x7fffffff;
+    for (int e = lane; e < c.experts; e += 64) {
+      const float v = choice[e];
+      if (v > value) { value = v; index = e; }     // (ascending e: the lowest index among equals)
+    }
+    wave_best(value, index);
+    if (index == 0x7fffffff) break;                // (nothing left to choose: refused on the host)
+    if (lane == k) mine = index;
+    if (lane == (index & 63)) choice[index] = -INFINITY;
+    sum += score[index];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
-  const float inverse = 1.0f / (sum + 1e-20f);
-  for (int k = 0; k < top; ++k) c.weights[(int64_t)t * c.experts + chosen[k]] = score[chosen[k]] * inverse;
+  if (mine >= 0) weights[mine] = score[mine] / (sum + 1e-20f);
 }
 
 BT_EXPORT int bt_route_call(void* stream, const RouteCall* c) {
@@ -114,14 +154,13 @@ BT_EXPORT int bt_route_call(void* stream, const RouteCall* c) {
     if (c->keep * (c->experts / c->groups) < c->top)
       BT_REFUSE("route: %d open groups of %d experts cannot give %d experts", c->keep, c->experts / c->groups, c->top);
   }
-  if (c->width <= 0 || c->width > 15360) BT_REFUSE("route: width %d outside 1..15360", c->width);
+  if (c->width <= 0) BT_REFUSE("route: width %d must be positive", c->width);
   if (!c->h || !c->W || !c->weights || (c->gate_w && !c->gate)) BT_REFUSE("route: missing operand");
   dim3 grid(c->tokens), block(ROUTE_THREADS);
-  const size_t lds = (size_t)c->width * sizeof(float);
   if (c->dtype == 0)
-    hipLaunchKernelGGL(route_kernel<float>, grid, block, lds, (hipStream_t)stream, *c);
+    hipLaunchKernelGGL(route_kernel<float>, grid, block, 0, (hipStream_t)stream, *c);
   else
-    hipLaunchKernelGGL(route_kernel<bf16_t>, grid, block, lds, (hipStream_t)stream, *c);
+    hipLaunchKernelGGL(route_kernel<bf16_t>, grid, block, 0, (hipStream_t)stream, *c);
   return bt_check_launch("route");
 }
 
@@ -152,7 +191,8 @@ __global__ void __launch_bounds__(256) gated_experts_kernel(GatedExpertsCall c) 
   T* hidden = static_cast<T*>(c.hidden) + (int64_t)t * c.ld_hidden;
   const float* weights = c.weights + (int64_t)t * (c.experts + c.identity);
   const int routed = c.experts * c.ff;
-  for (int col = threadIdx.x; col < c.hidden_cols; col += blockDim.x) {
+  // a token's columns are dealt to the work-groups of its row of the grid (a decode step has few tokens)
+  for (int col = blockIdx.y * blockDim.x + threadIdx.x; col < c.hidden_cols; col += gridDim.y * blockDim.x) {
     float out = 0.f;
     if (col < routed) {
       const int e = col / c.ff, i = col - e * c.ff;
@@ -172,7 +212,7 @@ __global__ void __launch_bounds__(256) gated_experts_kernel(GatedExpertsCall c) 
     float w = 0.f;
     for (int i = 0; i < c.identity; ++i) w += weights[c.experts + i];
     const T* h = static_cast<const T*>(c.h) + (int64_t)t * c.ldh;
-    for (int col = threadIdx.x; col < c.width; col += blockDim.x)
+    for (int col = blockIdx.y * blockDim.x + threadIdx.x; col < c.width; col += gridDim.y * blockDim.x)
       c.identity_out[(int64_t)t * c.width + col] = w != 0.f ? w * to_float(h[col]) : 0.f;
   }
 }
@@ -186,7 +226,10 @@ BT_EXPORT int bt_gated_experts_call(void* stream, const GatedExpertsCall* c) {
     BT_REFUSE("gated_experts: the rows do not hold the experts");
   if (!c->gu || !c->weights || !c->hidden || (c->identity_out && (!c->h || c->width <= 0)))
     BT_REFUSE("gated_experts: missing operand");
-  dim3 grid(c->tokens), block(256);
+  // about 1,024 columns a work-group, fewer work-groups a token where there are many tokens
+  int per_token = (c->hidden_cols + 1023) / 1024;
+  if (per_token > 64) per_token = 64;
+  dim3 grid(c->tokens, per_token), block(256);
   if (c->dtype == 0)
     hipLaunchKernelGGL(gated_experts_kernel<float>, grid, block, 0, (hipStream_t)stream, *c);
   else

@@ -75,21 +75,24 @@ __global__ void __launch_bounds__(HR_WAVES * 64) head_rotary_kernel(HeadRotaryCa
     keys = static_cast<T*>(c.kv.keys) + base;
     values = static_cast<T*>(c.kv.values) + base;
   }
-  for (int col = lane; col < hd; col += 64) {
-    float v = col < n ? row[col] : 0.f;
-    if (turned && col < c.rot_dims) {
-      const bool low = col < half;
-      const float angle = (float)pos * c.inv_freq[low ? col : col - half];
-      const float cs = cosf(angle), sn = sinf(angle);
-      v = low ? row[col] * cs - row[col + half] * sn : row[col] * cs + row[col - half] * sn;
-    }
+  auto store = [&](int col, float v) {
     if (is_q)
       q_out[col] = from_float<T>(v);
     else if (is_k)
       keys[key_offset(hd, pos, col)] = from_float<T>(v);
     else
       values[value_offset(hd, pos, col)] = from_float<T>(v);
-  }
+  };
+  // a lane takes a pair of channels: the angle's sine and cosine are computed once for both
+  if (turned)
+    for (int i = lane; i < half; i += 64) {
+      float sn, cs;
+      sincosf((float)pos * c.inv_freq[i], &sn, &cs);
+      const float u = row[i], v = row[i + half];
+      store(i, u * cs - v * sn);
+      store(i + half, v * cs + u * sn);
+    }
+  for (int col = (turned ? c.rot_dims : 0) + lane; col < hd; col += 64) store(col, col < n ? row[col] : 0.f);
 }
 
 BT_EXPORT int bt_head_rotary_call(void* stream, const HeadRotaryCall* c) {

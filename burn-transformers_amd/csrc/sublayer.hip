@@ -26,7 +26,22 @@ struct OutputNormCall {
   int64_t ld_cast;
   int kind;              // 0: layer norm (mean taken off, `beta` added), 1: RMS norm
   const float* beta;     // [width] or null
+  // The norm that reads the stream next, in the same pass over the row: next_out[t] = norm'(new x[t])
+  // (what the next sublayer multiplies by).  next_out null: none.
+  void* next_out;        // [tokens][next_ld] in the type `next_dtype`
+  int64_t next_ld;
+  int next_dtype;
+  int next_kind;
+  float next_eps;
+  const float* next_gamma;
+  const float* next_beta;   // or null
 };
+
+// y = N'(v) for one element, given the row's statistics
+__device__ __forceinline__ float next_norm(const OutputNormCall& c, float v, float mean, float rstd, int col) {
+  const float y = (v - mean) * rstd * c.next_gamma[col];
+  return c.next_beta ? y + c.next_beta[col] : y;
+}
 
 template <typename T>
 __global__ void __launch_bounds__(256) output_norm_kernel(OutputNormCall c) {
@@ -60,11 +75,26 @@ __global__ void __launch_bounds__(256) output_norm_kernel(OutputNormCall c) {
     if (c.beta) y += c.mult * c.beta[col];
     if (c.accumulate) y += xr[col];
     xr[col] = y;
+    row_buf[col] = y;         // (a thread's own columns: read back below by the same thread)
     if (cast) cast[(int64_t)t * c.ld_cast + col] = from_float<T>(y);
   }
   if (cast)
     for (int col = c.width + threadIdx.x; col < c.cast_cols; col += blockDim.x)
       cast[(int64_t)t * c.ld_cast + col] = from_float<T>(0.f);
+  if (c.next_out) {
+    float sum = 0.f;
+    if (c.next_kind == 0)
+      for (int col = threadIdx.x; col < c.width; col += blockDim.x) sum += row_buf[col];
+    const float next_mean = c.next_kind == 0 ? block_sum(sum, scratch) / (float)c.width : 0.f;
+    sum = 0.f;
+    for (int col = threadIdx.x; col < c.width; col += blockDim.x) sum += (row_buf[col] - next_mean) * (row_buf[col] - next_mean);
+    const float next_rstd = 1.0f / sqrtf(block_sum(sum, scratch) / (float)c.width + c.next_eps);
+    for (int col = threadIdx.x; col < c.width; col += blockDim.x) {
+      const float y = next_norm(c, row_buf[col], next_mean, next_rstd, col);
+      if (c.next_dtype == 0) static_cast<float*>(c.next_out)[(int64_t)t * c.next_ld + col] = y;
+      else static_cast<bf16_t*>(c.next_out)[(int64_t)t * c.next_ld + col] = (bf16_t)y;
+    }
+  }
 }
 
 // The same for rows of up to 256 * KMAX columns: a thread's columns live in registers and every load
@@ -112,12 +142,40 @@ __global__ void __launch_bounds__(256) output_norm_small_kernel(OutputNormCall c
     if (col < c.width) {
       const float y = v[k] * scale * g[k] + b[k] + xv[k];
       xr[col] = y;
+      v[k] = y;
       if (cast) cast[(int64_t)t * c.ld_cast + col] = from_float<T>(y);
+    } else {
+      v[k] = 0.f;
     }
   }
   if (cast)
     for (int col = c.width + threadIdx.x; col < c.cast_cols; col += blockDim.x)
       cast[(int64_t)t * c.ld_cast + col] = from_float<T>(0.f);
+  if (c.next_out) {           // the norm that reads the new row next, from the registers that hold it
+    float next_mean = 0.f;
+    if (c.next_kind == 0) {
+      float sum = 0.f;
+#pragma unroll
+      for (int k = 0; k < KMAX; ++k) sum += v[k];
+      next_mean = block_sum(sum, scratch) / (float)c.width;
+    }
+    float squares = 0.f;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const float d = threadIdx.x + 256 * k < c.width ? v[k] - next_mean : 0.f;
+      squares += d * d;
+    }
+    const float next_rstd = 1.0f / sqrtf(block_sum(squares, scratch) / (float)c.width + c.next_eps);
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int col = threadIdx.x + 256 * k;
+      if (col < c.width) {
+        const float y = next_norm(c, v[k], next_mean, next_rstd, col);
+        if (c.next_dtype == 0) static_cast<float*>(c.next_out)[(int64_t)t * c.next_ld + col] = y;
+        else static_cast<bf16_t*>(c.next_out)[(int64_t)t * c.next_ld + col] = (bf16_t)y;
+      }
+    }
+  }
 }
 
 template <typename T>
@@ -137,6 +195,8 @@ BT_EXPORT int bt_output_norm_call(void* stream, const OutputNormCall* c) {
   if (!c->x || !c->gamma || (c->n_delta > 0 && !c->delta)) BT_REFUSE("output_norm: missing operand");
   if (c->n_delta == 0 && c->accumulate) BT_REFUSE("output_norm: the stream's own rows cannot be added to themselves");
   if (c->kind != 0 && c->kind != 1) BT_REFUSE("output_norm: unknown kind of norm %d", c->kind);
+  if (c->next_out && (!c->next_gamma || c->next_ld < c->width || (c->next_kind != 0 && c->next_kind != 1)))
+    BT_REFUSE("output_norm: the norm that follows lacks its scale, its kind or room for its rows");
   if (c->cast && (c->cast_cols < c->width || c->ld_cast < c->cast_cols))
     BT_REFUSE("output_norm: a copy of %d columns in rows of %lld does not hold width %d", c->cast_cols,
               (long long)c->ld_cast, c->width);

@@ -87,7 +87,9 @@ class OutputNormCall(ctypes.Structure):
     _fields_ = [("cast_dtype", _c_int), ("n_delta", _c_int), ("tokens", _c_int), ("width", _c_int),
                 ("accumulate", _c_int), ("cast_cols", _c_int), ("eps", _c_float), ("mult", _c_float), ("x", _c_ptr),
                 ("delta", _c_ptr), ("delta_stride", _c_i64), ("ldd", _c_i64), ("bias", _c_ptr), ("gamma", _c_ptr),
-                ("cast", _c_ptr), ("ld_cast", _c_i64), ("kind", _c_int), ("beta", _c_ptr)]
+                ("cast", _c_ptr), ("ld_cast", _c_i64), ("kind", _c_int), ("beta", _c_ptr), ("next_out", _c_ptr),
+                ("next_ld", _c_i64), ("next_dtype", _c_int), ("next_kind", _c_int), ("next_eps", _c_float),
+                ("next_gamma", _c_ptr), ("next_beta", _c_ptr)]
     _step_fields_ = {"tokens": "tokens"}
 
 
@@ -1004,12 +1006,15 @@ def count_tokens(counts, rows, tokens):
 
 # --- norms of a sublayer's output, activations that are norms ---------------------------------
 
-def output_norm(x, gamma, eps, mult=1.0, delta=None, bias=None, accumulate=True, cast=None, kind="rms_norm", beta=None):
+def output_norm(x, gamma, eps, mult=1.0, delta=None, bias=None, accumulate=True, cast=None, kind="rms_norm", beta=None,
+                then=None):
     """x[t] (+)= mult * N(v) with v = sum(delta[:, t]) + bias (``delta`` float32 [splits, tokens, width]
     or [tokens, width]) and N the norm of ``kind``: v / sqrt(mean(v^2) + eps) * gamma, or for
     "layer_norm" (v - mean) / sqrt(var + eps) * gamma + beta; without ``delta`` the stream's own rows
     are normalised in place (``accumulate`` must then be False).  ``cast``: a tensor [tokens, >= width]
-    in the products' type that receives the new x (and zeros behind it)."""
+    in the products' type that receives the new x (and zeros behind it).  ``then``: (kind, gamma, beta,
+    eps, out) of the norm that reads the stream next; ``out`` [tokens, width] receives that norm of the
+    new x in the same pass."""
     tokens, width = x.shape
     if delta is None:
         n_delta, stride, ldd = 0, 0, 0
@@ -1023,7 +1028,11 @@ def output_norm(x, gamma, eps, mult=1.0, delta=None, bias=None, accumulate=True,
                            cast_cols=cast.shape[1] if cast is not None else 0, eps=eps, mult=mult, x=x.data_ptr(),
                            delta=_ptr(delta), delta_stride=stride, ldd=ldd, bias=_ptr(bias), gamma=gamma.data_ptr(),
                            cast=_ptr(cast), ld_cast=cast.stride(0) if cast is not None else 0,
-                           kind=NORM_KINDS[kind], beta=_ptr(beta)))
+                           kind=NORM_KINDS[kind], beta=_ptr(beta),
+                           next_out=then[4].data_ptr() if then else None, next_ld=then[4].stride(0) if then else 0,
+                           next_dtype=DTYPE_CODES[then[4].dtype] if then else 0, next_kind=NORM_KINDS[then[0]] if then else 0,
+                           next_eps=then[3] if then else 0.0, next_gamma=_ptr(then[1]) if then else None,
+                           next_beta=_ptr(then[2]) if then else None))
 
 
 def join_rows(x, y, out):

@@ -50,13 +50,28 @@ class ResidualStream:
         # the embedding's output, float32 [tokens, width], where the embedding keeps it for parts
         # that read it again later (``keep_origin``); None otherwise
         self.origin = None
+        # (norm, step, Delta, mult): x += mult * norm(Delta) that has not been done yet, because the
+        # norm that reads the stream next does it in the same kernel (``defer_output``)
+        self.pending_output = None
+
+    def defer_output(self, norm, step, delta, mult=1.0):
+        """x += mult * norm(delta), left for the next norm's ``apply`` to do in one kernel with its own
+        norm; whatever else touches the stream first does it alone (``flush``).  ``delta``'s buffers
+        must stay as they are until then."""
+        self.flush()
+        self.pending_output = (norm, step, delta, mult)
+        self.cast = None
+
+    def take_pending_output(self):
+        held, self.pending_output = self.pending_output, None
+        return held
 
     def operand(self, step):
         """The stream's rows as a product's operand: x itself in float32 models, its copy in the
         products' type otherwise."""
         if self.cast is not None:
             return self.cast
-        if self.pending is not None:
+        if self.pending is not None or self.pending_output is not None:
             self.flush()
         if step.dtype != self.x.dtype:
             raise ValueError("the residual stream has no copy in the products' type here: the part that "
@@ -64,7 +79,7 @@ class ResidualStream:
         return self.x
 
     def add(self, delta):
-        if self.pending is not None:
+        if self.pending is not None or self.pending_output is not None:
             self.flush()
         self.pending = delta
         self.cast = None            # x is about to change, its copy is not
@@ -91,6 +106,9 @@ class ResidualStream:
         if self.pending is not None:
             K.add_norm(self.x, None, None, None, 0.0, delta=self.pending.partials, bias=self.pending.bias)
             self.pending = None
+        if self.pending_output is not None:
+            norm, step, delta, mult = self.take_pending_output()
+            norm.add_output(self, step, delta, mult, keep_operand=False)
 
 
 def stream_product_splits(step, a, weight):

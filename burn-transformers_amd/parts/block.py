@@ -126,12 +126,13 @@ class SandwichNormBlock(Block):
         mixer = parts["mixer"]
         h = _apply(parts["mixer_norm"], stream, step, mixer.takes_deferred_norm)
         delta = mixer.forward(h, step, memory, output)
-        parts["mixer_post"].add_output(stream, step, delta if delta is not None else output.take(), keep_operand=False)
+        # what a sublayer adds is normalised by the kernel that normalises the stream for the next one
+        stream.defer_output(parts["mixer_post"], step, delta if delta is not None else output.take())
         if "ff" in parts:
             ff = parts["ff"]
             h = _apply(parts["ff_norm"], stream, step, ff.takes_deferred_norm)
             delta = ff.forward(h, step, output)
-            parts["ff_post"].add_output(stream, step, delta if delta is not None else output.take(), keep_operand=False)
+            stream.defer_output(parts["ff_post"], step, delta if delta is not None else output.take())
 
 
 @register("block", "transform")

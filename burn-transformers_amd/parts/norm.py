@@ -46,6 +46,14 @@ class _KernelNorm(Norm):
             out = K.Chunked.take(step, "norm.out" if rows is None else "norm.selected", count, self.width, step.dtype)     # for a part that only hands it to `gemm`
         else:
             out = step.buffer("norm.out" if rows is None else "norm.selected", count, self.width, step.dtype)
+        if stream.pending_output is not None:
+            if rows is None and not isinstance(out, K.Chunked):
+                # the norm of the last sublayer's output is still to join the stream: one kernel for both
+                post, post_step, delta, mult = stream.take_pending_output()
+                post.add_output(stream, post_step, delta, mult, keep_operand=False,
+                                then=(self.KIND, self.weight, self.bias, self.eps, out))
+                return out
+            stream.flush()
         pending = stream.pending
         K.add_norm(stream.x, out, self.weight, self.bias, self.eps, self.KIND,
                    delta=pending.partials if pending else None, bias=pending.bias if pending else None,
@@ -58,24 +66,26 @@ class _KernelNorm(Norm):
         return step.dtype_is_bf16 and K.Normalized.worth_it(rows, self.width)
 
     def deferred(self, stream, step):
-        if stream.pending is not None or not self.deferred_possible(step, stream.x.shape[0]):
+        if stream.pending is not None or stream.pending_output is not None or \
+                not self.deferred_possible(step, stream.x.shape[0]):
             return None
         return K.Normalized(stream.x, self.weight, self.bias, self.eps, self.KIND)
 
 
-    def add_output(self, stream, step, delta, mult=1.0, accumulate=True, keep_operand=True):
+    def add_output(self, stream, step, delta, mult=1.0, accumulate=True, keep_operand=True, then=None):
         """x (+)= mult * norm(v), v = the sublayer's output ``delta`` (a ``Delta``; None: the stream's
         own rows, normalised in place).  In a bfloat16 model the new rows are also left as the
         stream's copy in the products' type (``stream.operand``) unless ``keep_operand`` is False
-        (layers whose sublayers read a norm of the stream have no use for it)."""
-        if stream.pending is not None:
+        (layers whose sublayers read a norm of the stream have no use for it).  ``then``: the norm
+        that reads the stream next, computed in the same pass (``kernels.library.output_norm``)."""
+        if stream.pending is not None or stream.pending_output is not None:
             stream.flush()
         cast = None
         if keep_operand and step.dtype != stream.x.dtype:
             cast = step.buffer("stream.operand", stream.x.shape[0], operand_columns(self.width, step.dtype), step.dtype)
         K.output_norm(stream.x, self.weight, self.eps, mult, delta=delta.partials if delta is not None else None,
                       bias=delta.bias if delta is not None else None, accumulate=accumulate, cast=cast,
-                      kind=self.KIND, beta=self.bias)
+                      kind=self.KIND, beta=self.bias, then=then)
         stream.cast = cast
 
 

@@ -175,6 +175,22 @@ def test_norm_of_a_sublayers_output(width, kind):
     else:
         normed = v / torch.sqrt((v * v).mean(-1, keepdim=True) + 1e-4) * gamma.double()
     assert rel_err(stream, x.double() + 0.8 * normed) < 3e-6
+    # the same with the norm that reads the stream next done in the same pass
+    for then_kind, dt in (("layer_norm", torch.float32), ("rms_norm", torch.bfloat16), ("layer_norm", torch.bfloat16)):
+        stream = x.clone().to(DEV)
+        out = torch.full((rows, width + 8), float("nan"), dtype=dt, device=DEV)[:, :width]
+        g2, b2 = torch.randn(width, generator=gen), torch.randn(width, generator=gen)
+        K.output_norm(stream, gamma.to(DEV), 1e-4, 0.8, delta=delta.to(DEV), bias=bias.to(DEV), kind=kind,
+                      beta=beta.to(DEV) if kind == "layer_norm" else None,
+                      then=(then_kind, g2.to(DEV), b2.to(DEV) if then_kind == "layer_norm" else None, 1e-3, out))
+        y = x.double() + 0.8 * normed
+        assert rel_err(stream, y) < 3e-6
+        if then_kind == "layer_norm":
+            mean = y.mean(-1, keepdim=True)
+            want = (y - mean) / torch.sqrt(((y - mean) ** 2).mean(-1, keepdim=True) + 1e-3) * g2.double() + b2.double()
+        else:
+            want = y / torch.sqrt((y * y).mean(-1, keepdim=True) + 1e-3) * g2.double()
+        assert rel_err(out, want) < (3e-6 if dt == torch.float32 else 5e-3)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
