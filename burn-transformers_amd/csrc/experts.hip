@@ -55,17 +55,44 @@ __global__ void __launch_bounds__(ROUTE_THREADS) route_kernel(RouteCall c) {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* h = static_cast<const T*>(c.h) + (int64_t)t * c.ldh;
   const int outputs = c.experts + (c.gate_w ? 1 : 0);
+  // the corrections of this lane's first experts are asked for now, with the first batch's loads
+  float early_correction[4] = {0.f, 0.f, 0.f, 0.f};
+  if (wave == 0 && c.correction)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (lane + 64 * j < c.experts) early_correction[j] = c.correction[lane + 64 * j];
+  float gate_value = 0.f;
   for (int first = 0; first < outputs; first += ROUTE_BATCH) {
     float sums[ROUTE_BATCH];
+    const float* rows[ROUTE_BATCH];                 // an output beyond the last reads the last one's row and is dropped
 #pragma unroll
-    for (int j = 0; j < ROUTE_BATCH; ++j) sums[j] = 0.f;
-    for (int col = threadIdx.x; col < c.width; col += ROUTE_THREADS) {
-      const float x = to_float(h[col]);
+    for (int j = 0; j < ROUTE_BATCH; ++j) {
+      sums[j] = 0.f;
+      const int e = first + j < outputs ? first + j : outputs - 1;
+      rows[j] = e < c.experts ? c.W + (int64_t)e * c.width : c.gate_w;
+    }
+    // four columns a thread and turn, none of the loads behind a branch of its own: all of a turn's
+    // loads are in flight together (behind branches they are waited for one by one)
+    for (int col0 = threadIdx.x; col0 < c.width; col0 += 4 * ROUTE_THREADS) {
+      int cc[4];
+      float xs[4];
 #pragma unroll
-      for (int j = 0; j < ROUTE_BATCH; ++j) {
-        const int e = first + j;
-        if (e < outputs) sums[j] = fmaf((e < c.experts ? c.W + (int64_t)e * c.width : c.gate_w)[col], x, sums[j]);
+      for (int u = 0; u < 4; ++u) {
+        const int col = col0 + u * ROUTE_THREADS;
+        cc[u] = col < c.width ? col : 0;
+        xs[u] = to_float(h[cc[u]]);
       }
+      float ws[ROUTE_BATCH][4];
+#pragma unroll
+      for (int j = 0; j < ROUTE_BATCH; ++j)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) ws[j][u] = rows[j][cc[u]];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) xs[u] = col0 + u * ROUTE_THREADS < c.width ? xs[u] : 0.f;
+#pragma unroll
+      for (int j = 0; j < ROUTE_BATCH; ++j)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sums[j] = fmaf(ws[j][u], xs[u], sums[j]);
     }
 #pragma unroll
     for (int j = 0; j < ROUTE_BATCH; ++j) {
@@ -78,11 +105,12 @@ __global__ void __launch_bounds__(ROUTE_THREADS) route_kernel(RouteCall c) {
       for (int w = 0; w < ROUTE_THREADS / 64; ++w) sum += partial[w][threadIdx.x];
       const int e = first + threadIdx.x;
       if (e < c.experts) score[e] = sum;
-      else c.gate[t] = 1.0f / (1.0f + expf(-sum));
+      else gate_value = sum;                       // (stored at the end: nothing waits for a store meanwhile)
     }
     __syncthreads();
   }
   if (wave != 0) return;
+  if (c.gate_w && (int)threadIdx.x == (outputs - 1) % ROUTE_BATCH) c.gate[t] = 1.0f / (1.0f + expf(-gate_value));
   float top_logit = -INFINITY;
   for (int e = lane; e < c.experts; e += 64) top_logit = fmaxf(top_logit, score[e]);
   top_logit = wave_max(top_logit);
@@ -90,11 +118,10 @@ __global__ void __launch_bounds__(ROUTE_THREADS) route_kernel(RouteCall c) {
   for (int e = lane; e < c.experts; e += 64) total += expf(score[e] - top_logit);
   total = wave_sum(total);
   float* weights = c.weights + (int64_t)t * c.experts;
-  for (int e = lane; e < c.experts; e += 64) {     // a lane keeps to its own experts: no other lane reads them yet
+  for (int e = lane, j = 0; e < c.experts; e += 64, ++j) {     // a lane keeps to its own experts: no other lane reads them yet
     const float s = expf(score[e] - top_logit) / total;
     score[e] = s;
-    choice[e] = s + (c.correction ? c.correction[e] : 0.f);
-    weights[e] = 0.f;
+    choice[e] = s + (c.correction ? (j < 4 ? early_correction[j < 4 ? j : 0] : c.correction[e]) : 0.f);
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -124,24 +151,24 @@ __global__ void __launch_bounds__(ROUTE_THREADS) route_kernel(RouteCall c) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
   float sum = 0.f;
-  int mine = -1;                                   // lane k keeps the k-th chosen expert
   for (int k = 0; k < c.top; ++k) {
     float value = -INFINITY;
     int index = 0x7fffffff;
     for (int e = lane; e < c.experts; e += 64) {
       const float v = choice[e];
-      if (v > value) { value = v; index = e; }     // (ascending e: the lowest index among equals)
+      if (v > value && v != INFINITY) { value = v; index = e; }     // (ascending e: the lowest index among equals; +inf: taken)
     }
     wave_best(value, index);
     if (index == 0x7fffffff) break;                // (nothing left to choose: refused on the host)
-    if (lane == k) mine = index;
-    if (lane == (index & 63)) choice[index] = -INFINITY;
+    if (lane == (index & 63)) choice[index] = INFINITY;            // taken: its owner marks it
     sum += score[index];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
-  if (mine >= 0) weights[mine] = score[mine] / (sum + 1e-20f);
+  // the one store of a lane's experts: the chosen ones' scores over their sum, zero elsewhere
+  const float inverse = 1.0f / (sum + 1e-20f);
+  for (int e = lane; e < c.experts; e += 64) weights[e] = choice[e] == INFINITY ? score[e] * inverse : 0.f;
 }
 
 BT_EXPORT int bt_route_call(void* stream, const RouteCall* c) {

@@ -105,24 +105,63 @@ __global__ void __launch_bounds__(256) output_norm_small_kernel(OutputNormCall c
   __shared__ float scratch[32];
   const int t = blockIdx.x;
   float* xr = c.x + (int64_t)t * c.width;
+  // Every load of a thread is issued before the first is used and none stands behind a branch of its
+  // own (columns beyond the row and partial sums beyond the last are read from a valid place and
+  // dropped): loads behind branches, or in a loop of unknown length, are waited for one by one, and
+  // a row then costs as many round trips to memory as it has of them (measured: 14 us for 16 of them).
   float v[KMAX], xv[KMAX], g[KMAX], b[KMAX];
+  int cc[KMAX];
+  bool in_row[KMAX];
 #pragma unroll
   for (int k = 0; k < KMAX; ++k) {
     const int col = threadIdx.x + 256 * k;
-    v[k] = xv[k] = g[k] = b[k] = 0.f;
-    if (col < c.width) {
-      g[k] = c.gamma[col];
-      if (c.beta) b[k] = c.mult * c.beta[col];
-      if (c.n_delta == 0) {
-        v[k] = xr[col];
-      } else {
-        if (c.accumulate) xv[k] = xr[col];
-        float sum = c.bias ? c.bias[col] : 0.f;
-        for (int s = 0; s < c.n_delta; ++s) sum += c.delta[s * c.delta_stride + (int64_t)t * c.ldd + col];
-        v[k] = sum;
-      }
-    }
+    in_row[k] = col < c.width;
+    cc[k] = in_row[k] ? col : 0;
   }
+  const float* beta = c.beta ? c.beta : c.gamma;           // (read in any case, used only where there is one)
+  const float* bias = c.bias ? c.bias : c.gamma;
+  const float* gamma2 = c.next_out ? c.next_gamma : c.gamma;
+  const float* beta2 = c.next_out && c.next_beta ? c.next_beta : c.gamma;
+  float g2[KMAX], b2[KMAX];
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    g2[k] = gamma2[cc[k]];
+    b2[k] = beta2[cc[k]];
+    g[k] = c.gamma[cc[k]];
+    b[k] = beta[cc[k]];
+    xv[k] = xr[cc[k]];
+    v[k] = bias[cc[k]];
+  }
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    b[k] = c.beta ? c.mult * b[k] : 0.f;
+    v[k] = c.bias ? v[k] : 0.f;
+  }
+  if (c.n_delta == 0) {
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) { v[k] = xv[k]; xv[k] = 0.f; }
+  } else {
+    const float* row = c.delta + (int64_t)t * c.ldd;
+    for (int s0 = 0; s0 < c.n_delta; s0 += 4) {            // four partial sums at a time, all their loads together
+      float part[4][KMAX];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int sc = s0 + u < c.n_delta ? s0 + u : c.n_delta - 1;
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) part[u][k] = row[sc * c.delta_stride + cc[k]];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k) v[k] += s0 + u < c.n_delta ? part[u][k] : 0.f;
+    }
+    if (!c.accumulate)
+#pragma unroll
+      for (int k = 0; k < KMAX; ++k) xv[k] = 0.f;
+  }
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k)
+    if (!in_row[k]) v[k] = xv[k] = g[k] = b[k] = 0.f;
   float partial = 0.f;
   if (c.kind == 0) {          // a layer norm: the mean first, then the squared distances from it
 #pragma unroll
@@ -170,7 +209,7 @@ __global__ void __launch_bounds__(256) output_norm_small_kernel(OutputNormCall c
     for (int k = 0; k < KMAX; ++k) {
       const int col = threadIdx.x + 256 * k;
       if (col < c.width) {
-        const float y = next_norm(c, v[k], next_mean, next_rstd, col);
+        const float y = (v[k] - next_mean) * next_rstd * g2[k] + (c.next_beta ? b2[k] : 0.f);
         if (c.next_dtype == 0) static_cast<float*>(c.next_out)[(int64_t)t * c.next_ld + col] = y;
         else static_cast<bf16_t*>(c.next_out)[(int64_t)t * c.next_ld + col] = (bf16_t)y;
       }

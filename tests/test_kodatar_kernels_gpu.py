@@ -156,11 +156,11 @@ def test_gated_experts_activation(dtype, experts, ff, shared, identity):
         assert rel_err(identity_out, total * h.double()) < 2e-6
 
 
+@pytest.mark.parametrize("rows", [9, 70])          # a wave a row up to 64 rows, a work-group a row beyond
 @pytest.mark.parametrize("width", [40, 256, 1500, 2600])
 @pytest.mark.parametrize("kind", ["layer_norm", "rms_norm"])
-def test_norm_of_a_sublayers_output(width, kind):
+def test_norm_of_a_sublayers_output(width, kind, rows):
     gen = torch.Generator().manual_seed(width)
-    rows = 9
     x = torch.randn(rows, width, generator=gen)
     delta = torch.randn(3, rows, width, generator=gen) + 0.7
     bias = torch.randn(width, generator=gen)
