@@ -79,6 +79,7 @@ class RotaryAttention(CausalSelfAttention):
             raise ValueError(f"rotary attention: the bfloat16 kernels take heads of up to 128, not {self.head_dim}; "
                              f"load the model with dtype float32")
         self.plain_only = False
+        self.plain_decode = bf16 and self.heads // self.kv_heads > 16
         self.n_q, self.n_kv = self.heads * self.head_dim, self.kv_heads * self.head_dim
         self.fused_cols = (self.heads + self.kv_heads) * self.dim + self.kv_heads * self.vdim
         self.qkv_weight = torch.cat([tensors["q_weight"], tensors["k_weight"], tensors["v_weight"]]).contiguous()
@@ -108,7 +109,7 @@ class RotaryAttention(CausalSelfAttention):
         q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
         K.head_rotary(fused, self.heads, self.kv_heads, self.dim, self.vdim, self.rot_dims, self.inv_freq,
                       self.q_norm, self.k_norm, self.eps, q, step.tok_seq, step.tok_pos, kv, step.dtype)
-        if step.decode and step.dtype_is_bf16 and K.Chunked.wanted(tokens) and self.heads // self.kv_heads <= 16:
+        if step.decode and step.dtype_is_bf16 and K.Chunked.wanted(tokens) and not self.plain_decode:
             mixed = K.Chunked.take(step, "attention.mixed", tokens, self.n_q, step.dtype)
         else:
             mixed = step.buffer("attention.mixed", tokens, self.n_q, step.dtype)
@@ -118,5 +119,6 @@ class RotaryAttention(CausalSelfAttention):
         args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
                                 self.heads, step.n_seqs, step.max_count, self.scale, self.window, partial,
                                 chunk=self.chunk)
-        K.attention(args, step.dtype, step.decode)
+        # (the bfloat16 decode kernel takes up to 16 query heads on a cached head; beyond, the plain kernel)
+        K.attention(args, step.dtype, step.decode, impl="plain" if self.plain_decode and step.decode else "auto")
         stream.add_product(step, mixed, self.out_weight, None, packed=self.out_packed)

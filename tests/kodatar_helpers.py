@@ -58,7 +58,9 @@ LONG = model_config([layer(mixer(2, 1, 128, 64, 0.09, rot_dims=64, base=250000.0
                                  chunk=448), moe(4, 32, 2, shared=32)),
                      layer(mixer(4, 2, 48, 48, 0.14, rot_dims=48, base=10000.0), moe(4, 32, 1, identity=1))],
                     width=96, vocab=151, loop=(0, 2, 2))
-CONFIGS = {"basic": (BASIC, 1), "odd": (ODD, 2), "attention": (ATTENTION_ONLY, 3), "causal": (FULL_CAUSAL, 4),
+# more query heads on a cached head than a decode tile takes, and one cached head for all
+MANY_HEADS = model_config([layer(mixer(20, 1, 16, 16, 0.25, rot_dims=16, chunk=48), moe(2, 16, 1, shared=8))], width=48, vocab=71)
+CONFIGS = {"many_heads": (MANY_HEADS, 9), "basic": (BASIC, 1), "odd": (ODD, 2), "attention": (ATTENTION_ONLY, 3), "causal": (FULL_CAUSAL, 4),
            "experts": (EXPERTS_PLAIN, 5), "experts_full": (EXPERTS_FULL, 6), "loop": (LOOP_ONLY, 7), "long": (LONG, 8)}
 
 _weights, _models = {}, {}

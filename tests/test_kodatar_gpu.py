@@ -79,7 +79,8 @@ def test_residual_stream_after_every_run_of_a_layer():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,length,tail", [("basic", 80, 40), ("odd", 110, 20), ("attention", 140, 80), ("loop", 9, 8)])
+@pytest.mark.parametrize("name,length,tail", [("basic", 80, 40), ("odd", 110, 20), ("attention", 140, 80), ("loop", 9, 8),
+                                              ("many_heads", 100, 30)])
 def test_prompt_then_token_by_token(name, dtype, length, tail):
     """The last tokens one by one through the cache give what the whole prompt gives; the tails pass
     over chunk edges."""
@@ -263,3 +264,56 @@ def test_folder_round_trip_and_replay(tmp_path):
     for step, row in ((1, 40), (2, 41)):
         got = torch.from_numpy(np.fromfile(tmp_path / "out" / f"{step}.f32", dtype="<f4").reshape(1, -1)).double()
         check(got, want_a[row:row + 1], "float32", f"replayed step {step}")
+
+
+def test_command_line(capsys, tmp_path):
+    """The command line takes the family by config.json: random weights written from a configuration,
+    then greedy tokens for two prompts, then sampled ones with the prompts fed in portions."""
+    import json
+    from burn_transformers_amd.cli import main
+    config, seed = CONFIGS["basic"]
+    cfg_path = tmp_path / "cfg.json"
+    cfg_path.write_text(json.dumps(config))
+    prompts = prompts_for("basic", [6, 30], seed=60)
+    text = ";".join(",".join(str(t) for t in p) for p in prompts)
+    assert main([str(tmp_path / "made"), text, "5", "--dtype", "float32", "--json", "--random-weights", str(cfg_path),
+                 "--weights-seed", str(seed)]) == 0
+    lines = [json.loads(line) for line in capsys.readouterr().out.strip().splitlines()]
+    weights = weights_for("basic")
+    assert [line["token_ids"] for line in lines] == [plain.greedy(p, weights, config, 5) for p in prompts]
+    assert main([str(tmp_path / "made"), text, "4", "--temperature", "0.7", "--seed", "5", "--prefill-chunk-size", "4"]) == 0
+
+
+def test_trace_runner_as_a_program(tmp_path):
+    """bin/trace_run in a process of its own, in both number formats: a batch of two prompts, then
+    both decoded together, one of them ending first."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    config = CONFIGS["odd"][0]
+    weights = weights_for("odd", dtype="bfloat16")          # (routing that hangs on no close call, for both formats)
+    os.makedirs(tmp_path / "model")
+    (tmp_path / "model" / "config.json").write_text(json.dumps(config))
+    bt.write_safetensors(str(tmp_path / "model" / "model.safetensors"), {k: v.to(torch.bfloat16) for k, v in weights.items()})
+    a, b = prompts_for("odd", [70, 12], seed=22)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": a[:66], "want": [65]}, {"id": "y", "tokens": b[:10], "want": [0, 9]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": a[66:67], "want": [0]}, {"id": "y", "tokens": b[10:11], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": a[67:68], "want": [0]}, {"id": "y", "tokens": b[11:12], "want": [0]}], "end": ["y"]},
+             {"step": 3, "entries": [{"id": "x", "tokens": a[68:69], "want": [0]}], "end": ["x"]}]
+    want_a, want_b = plain.forward(a, weights, config), plain.forward(b, weights, config)
+    expected = {0: [want_a[65], want_b[0], want_b[9]], 1: [want_a[66]], 2: [want_a[67], want_b[11]], 3: [want_a[68]]}
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for dtype in DTYPES:
+        out = tmp_path / ("out_" + dtype)
+        done = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(tmp_path / "model"),
+                               "--dtype", dtype, "--out", str(out), "--max-tokens", "100"],
+                              input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+        assert done.returncode == 0, done.stderr[-2000:]
+        assert [line for line in done.stdout.splitlines() if line.startswith("done")] == [f"done {i}" for i in range(4)]
+        for step, rows in expected.items():
+            got = torch.from_numpy(np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(len(rows), -1)).double()
+            want = torch.stack(rows)
+            bound = tolerance(dtype, want_a)
+            assert float((got - want).abs().max()) <= bound, (dtype, step)
