@@ -128,8 +128,9 @@ class CacheLedger:
         for group in range(self.n_groups):
             held = self.held_blocks[group][slot]
             if RELEASED in held[self.first_kept(group, length):keep]:
-                raise ValueError(f"slot {slot} cannot be rewound to {length} tokens: a layer with a window of "
-                                 f"{self.windows[group]} (or chunks of {self.chunks[group]}) has given the blocks before it back already")
+                reach = f"a window of {self.windows[group]}" if self.windows[group] > 0 else f"chunks of {self.chunks[group]}"
+                raise ValueError(f"slot {slot} cannot be rewound to {length} tokens: a layer with {reach} "
+                                 f"has given the blocks before it back already")
         for group in range(self.n_groups):
             held = self.held_blocks[group][slot]
             while len(held) > keep:

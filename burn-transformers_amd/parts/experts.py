@@ -22,8 +22,10 @@ other (the shared expert's last), a kernel that applies silu(gate) * up times th
 that expert (zero where it was not chosen, the sigmoid gate for the shared expert), and ONE product
 with the down matrices laid side by side, which so sums the weighted outputs.  No token is moved
 and nothing depends on the host knowing the choice, so the step is a fixed list of kernels like
-every other; the price is that every expert multiplies every token (see DESIGN.md's section on
-this part for when that is a good trade and when it is not).
+every other; the price is that every expert multiplies every token.  In decode steps that costs
+little once tokens * top reaches the number of experts (all matrices are read anyway); a prompt does
+experts / top times the routed arithmetic, which a grouped product over tokens sorted by expert
+would save.
 """
 
 import torch

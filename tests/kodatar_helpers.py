@@ -53,8 +53,8 @@ EXPERTS_FULL = model_config([layer(mixer(1, 1, 16, 16, 0.25), moe(9, 8, 3, ident
                             width=32, vocab=61)
 LOOP_ONLY = model_config([layer(mixer(2, 2, 16, 16, 0.25, rot_dims=8))], width=32, vocab=61, loop=(0, 1, 4))
 # heads of 128, chunks that span several blocks: keys far back and at block borders
-LONG = model_config([layer(mixer(2, 1, 128, 64, 0.09, rot_dims=64, base=250000.0, scaling={"factor": 8.0, "low": 1.0,
-                                                                                           "high": 4.0, "original": 256},
+LONG = model_config([layer(mixer(2, 1, 128, 64, 0.09, rot_dims=64, base=300000.0, scaling={"factor": 6.0, "low": 1.0,
+                                                                                           "high": 5.0, "original": 256},
                                  chunk=448), moe(4, 32, 2, shared=32)),
                      layer(mixer(4, 2, 48, 48, 0.14, rot_dims=48, base=10000.0), moe(4, 32, 1, identity=1))],
                     width=96, vocab=151, loop=(0, 2, 2))

@@ -52,20 +52,20 @@ def test_a_folded_norm_is_worth_it_by_rows_and_width():
 
 # --- the runs a decode step's keys are cut into, and the classes of context ---------------------
 
-def _runs(monkeypatch, n_seqs, context_limit, kv_heads=25, head_dim=64, bf16=True, window=0, decode=True, units=256):
+def _runs(monkeypatch, n_seqs, context_limit, kv_heads=25, head_dim=64, bf16=True, window=0, decode=True, units=256, chunk=0):
     from types import SimpleNamespace
     from burn_transformers_amd.parts import attention
     monkeypatch.setattr(attention, "compute_units", lambda device: units)
-    mixer = SimpleNamespace(kv_heads=kv_heads, head_dim=head_dim, window=window)
+    mixer = SimpleNamespace(kv_heads=kv_heads, head_dim=head_dim, window=window, chunk=chunk)
     step = SimpleNamespace(decode=decode, context_limit=context_limit, dtype_is_bf16=bf16, n_seqs=n_seqs)
     return attention.CausalSelfAttention.decode_runs(mixer, step, "cuda:0")
 
 
-def _prompt_runs(monkeypatch, capacity, n_seqs, context_limit, heads=25, head_dim=64, bf16=True, window=0, units=256):
+def _prompt_runs(monkeypatch, capacity, n_seqs, context_limit, heads=25, head_dim=64, bf16=True, window=0, units=256, chunk=0):
     from types import SimpleNamespace
     from burn_transformers_amd.parts import attention
     monkeypatch.setattr(attention, "compute_units", lambda device: units)
-    mixer = SimpleNamespace(heads=heads, head_dim=head_dim, window=window, plain_only=False)
+    mixer = SimpleNamespace(heads=heads, head_dim=head_dim, window=window, chunk=chunk, plain_only=False)
     step = SimpleNamespace(decode=False, context_limit=context_limit, dtype_is_bf16=bf16, n_seqs=n_seqs,
                            token_capacity=capacity)
     return attention.CausalSelfAttention.prompt_runs(mixer, step, "cuda:0")
@@ -88,6 +88,7 @@ def test_prompt_runs_for_chunks_behind_long_contexts(monkeypatch):
     assert _prompt_runs(monkeypatch, 256, 1, 8192, bf16=False) == 1
     assert _prompt_runs(monkeypatch, 256, 1, 8192, head_dim=32) == 1
     assert _prompt_runs(monkeypatch, 256, 1, 8192, window=512) == 1
+    assert _prompt_runs(monkeypatch, 256, 1, 8192, chunk=512) == 1
     assert _prompt_runs(monkeypatch, 256, 1, 8192, heads=4) == 8   # few heads: the runs are what fills the chip
 
 
@@ -105,6 +106,7 @@ def test_decode_runs_at_measured_sizes(monkeypatch):
     assert _runs(monkeypatch, 8, 1024, bf16=False) == 1
     # a window bounds the keys a query reads; steps with prompt tokens are never cut
     assert _runs(monkeypatch, 1, 8192, window=512) == 1
+    assert _runs(monkeypatch, 1, 8192, chunk=512) == 1          # so do chunks
     assert _runs(monkeypatch, 1, 8192, decode=False) == 1
 
 
