@@ -31,7 +31,7 @@ would save.
 import torch
 
 from ..kernels import library as K
-from .base import Delta, FeedForward, operand_columns, packed_for_stream, pad_columns, stream_product_splits
+from .base import Delta, FeedForward, operand_columns, packed_for_stream, pad_columns, pad_rows, stream_product_splits
 from .registry import register
 
 
@@ -82,7 +82,8 @@ class RoutedExperts(FeedForward):
         dtype = rows[0].dtype
         self.inner = self.experts * self.ff + self.shared_ff
         self.hidden_cols = operand_columns(self.inner, dtype)
-        self.in_weight = torch.cat(rows).contiguous()                                        # [2 * inner, width]
+        self.fused_cols = operand_columns(2 * self.inner, dtype)      # (rows of the fused product's output start where 16-byte stores may)
+        self.in_weight = pad_rows(torch.cat(rows), self.fused_cols)                           # [2 * inner (+ zero rows), width]
         self.down_weight = pad_columns(torch.cat(columns, dim=1), self.hidden_cols)           # [width, inner (+ zeros)]
         on_gpu = self.in_weight.is_cuda
         self.in_packed = K.PackedWeight(self.in_weight) if on_gpu else None
@@ -96,7 +97,7 @@ class RoutedExperts(FeedForward):
         weights = step.buffer("experts.weights", tokens, self.outputs, "float32")
         mix = step.buffer("experts.mix", tokens, 1, "float32") if self.shared_ff else None
         K.route(h, self.router, self.correction, self.top, self.groups, self.keep, weights, self.shared_mix, mix)
-        fused = step.buffer("experts.fused", tokens, 2 * self.inner, step.dtype)
+        fused = step.buffer("experts.fused", tokens, self.fused_cols, step.dtype)
         K.gemm(h, self.in_weight, K.epilogue_store(fused), packed=self.in_packed)
         hidden = step.buffer("experts.hidden", tokens, self.hidden_cols, step.dtype)
         splits = stream_product_splits(step, hidden, self.down_weight)

@@ -75,10 +75,8 @@ class RotaryAttention(CausalSelfAttention):
         self.head_dim = (max(self.dim, self.vdim) + 15) // 16 * 16
         if self.head_dim > 256:
             raise ValueError(f"rotary attention: heads of {max(self.dim, self.vdim)} are beyond 256, the most any kernel here takes")
-        if bf16 and self.head_dim > 128:
-            raise ValueError(f"rotary attention: the bfloat16 kernels take heads of up to 128, not {self.head_dim}; "
-                             f"load the model with dtype float32")
-        self.plain_only = False
+        # the MFMA kernels take heads of up to 128 in bfloat16; larger ones run on the plain attention kernel
+        self.plain_only = bf16 and self.head_dim > 128
         self.plain_decode = bf16 and self.heads // self.kv_heads > 16
         self.n_q, self.n_kv = self.heads * self.head_dim, self.kv_heads * self.head_dim
         self.fused_cols = (self.heads + self.kv_heads) * self.dim + self.kv_heads * self.vdim
@@ -109,16 +107,17 @@ class RotaryAttention(CausalSelfAttention):
         q = step.buffer("attention.q", tokens, self.n_q, step.dtype)
         K.head_rotary(fused, self.heads, self.kv_heads, self.dim, self.vdim, self.rot_dims, self.inv_freq,
                       self.q_norm, self.k_norm, self.eps, q, step.tok_seq, step.tok_pos, kv, step.dtype)
-        if step.decode and step.dtype_is_bf16 and K.Chunked.wanted(tokens) and not self.plain_decode:
+        plain = self.plain_only or (self.plain_decode and step.decode)
+        if step.decode and step.dtype_is_bf16 and K.Chunked.wanted(tokens) and not plain:
             mixed = K.Chunked.take(step, "attention.mixed", tokens, self.n_q, step.dtype)
         else:
             mixed = step.buffer("attention.mixed", tokens, self.n_q, step.dtype)
-        partial, runs = None, self.decode_runs(step, h.device)
+        partial, runs = None, 1 if plain else self.decode_runs(step, h.device)
         if runs > 1:
             partial = step.buffer("attention.partial", step.n_seqs * self.heads * runs, self.head_dim + 2, "float32")
         args = K.attention_args(q, mixed, kv, step.tok_seq, step.tok_pos, step.seq_off, step.seq_start,
                                 self.heads, step.n_seqs, step.max_count, self.scale, self.window, partial,
                                 chunk=self.chunk)
         # (the bfloat16 decode kernel takes up to 16 query heads on a cached head; beyond, the plain kernel)
-        K.attention(args, step.dtype, step.decode, impl="plain" if self.plain_decode and step.decode else "auto")
+        K.attention(args, step.dtype, step.decode, impl="plain" if plain else "auto")
         stream.add_product(step, mixed, self.out_weight, None, packed=self.out_packed)

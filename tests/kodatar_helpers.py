@@ -60,7 +60,9 @@ LONG = model_config([layer(mixer(2, 1, 128, 64, 0.09, rot_dims=64, base=300000.0
                     width=96, vocab=151, loop=(0, 2, 2))
 # more query heads on a cached head than a decode tile takes, and one cached head for all
 MANY_HEADS = model_config([layer(mixer(20, 1, 16, 16, 0.25, rot_dims=16, chunk=48), moe(2, 16, 1, shared=8))], width=48, vocab=71)
-CONFIGS = {"many_heads": (MANY_HEADS, 9), "basic": (BASIC, 1), "odd": (ODD, 2), "attention": (ATTENTION_ONLY, 3), "causal": (FULL_CAUSAL, 4),
+# heads wider than any MFMA attention kernel's (the plain attention kernel runs them), an odd feed-forward
+WIDE_HEADS = model_config([layer(mixer(2, 1, 144, 20, 0.08, rot_dims=100, chunk=30), moe(3, 5, 2, shared=3))], width=32, vocab=53)
+CONFIGS = {"wide_heads": (WIDE_HEADS, 10), "many_heads": (MANY_HEADS, 9), "basic": (BASIC, 1), "odd": (ODD, 2), "attention": (ATTENTION_ONLY, 3), "causal": (FULL_CAUSAL, 4),
            "experts": (EXPERTS_PLAIN, 5), "experts_full": (EXPERTS_FULL, 6), "loop": (LOOP_ONLY, 7), "long": (LONG, 8)}
 
 _weights, _models = {}, {}

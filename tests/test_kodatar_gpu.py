@@ -80,7 +80,7 @@ def test_residual_stream_after_every_run_of_a_layer():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name,length,tail", [("basic", 80, 40), ("odd", 110, 20), ("attention", 140, 80), ("loop", 9, 8),
-                                              ("many_heads", 100, 30)])
+                                              ("many_heads", 100, 30), ("wide_heads", 90, 40)])
 def test_prompt_then_token_by_token(name, dtype, length, tail):
     """The last tokens one by one through the cache give what the whole prompt gives; the tails pass
     over chunk edges."""
