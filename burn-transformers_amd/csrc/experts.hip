@@ -12,7 +12,7 @@
 // Ties between equal scores go to the lower index.
 #include "host.h"
 
-#define ROUTE_THREADS 256
+#define ROUTE_THREADS 1024
 #define ROUTE_MAX_EXPERTS 1024
 
 struct RouteCall {
@@ -30,8 +30,6 @@ struct RouteCall {
   float* gate;              // [tokens]: sigmoid(gate_w . h), or null
 };
 
-#define ROUTE_BATCH 16          // router outputs whose sums a thread carries at once
-
 // The best (value, index) of a wave; among equal values the lowest index.  Every lane gets it.
 __device__ __forceinline__ void wave_best(float& value, int& index) {
 #pragma unroll
@@ -42,75 +40,74 @@ __device__ __forceinline__ void wave_best(float& value, int& index) {
   }
 }
 
-// One work-group per token.  Logits: a thread takes the columns t, t + 256, ... of the row and carries
-// the sums of ROUTE_BATCH outputs at once, so that all loads of a batch are in flight together (a
-// decode step has few tokens: one round trip to memory is the kernel's time); the sums meet through
-// wave reductions and LDS.  Everything after the logits is the first wave's alone, the experts dealt
-// to its lanes, maxima and choices as wave reductions: no barrier, no serial scan.
+// One work-group of sixteen waves per token.  Logits: a wave takes whole outputs (two at a time, the
+// outputs dealt round the waves), its lanes the columns, sixteen a turn; nothing of a turn's loads stands
+// behind a branch of its own, so all of them are in flight together, every wave's at once: the
+// logits cost one round trip to memory and a wave reduction, and no sum crosses waves.  (Columns
+// dealt to the threads and sixteen outputs' sums met through LDS, batch after batch, took 6 us a batch
+// of sixteen outputs: a decode step has few tokens, and a kernel's time is the chain of its waits.)
+// Everything after the logits is the first wave's alone, the experts dealt to its lanes, maxima and
+// choices as wave reductions: no barrier, no serial scan.
+#define ROUTE_WAVES (ROUTE_THREADS / 64)
+#define ROUTE_OUTPUTS 2         // outputs whose sums a wave carries at once
+#define ROUTE_COLUMNS 16        // columns of a lane and turn
+
 template <typename T>
 __global__ void __launch_bounds__(ROUTE_THREADS) route_kernel(RouteCall c) {
-  __shared__ float partial[ROUTE_THREADS / 64][ROUTE_BATCH];
   __shared__ float score[ROUTE_MAX_EXPERTS];      // logits, then softmax scores
-  __shared__ float choice[ROUTE_MAX_EXPERTS];     // scores with the correction; -inf once taken or shut out
-  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ float choice[ROUTE_MAX_EXPERTS];     // scores with the correction; +inf once taken, -inf where shut out
+  __shared__ float gate_sum;
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const T* h = static_cast<const T*>(c.h) + (int64_t)t * c.ldh;
   const int outputs = c.experts + (c.gate_w ? 1 : 0);
-  // the corrections of this lane's first experts are asked for now, with the first batch's loads
+  // the corrections of this lane's first experts are asked for now, with the first loads
   float early_correction[4] = {0.f, 0.f, 0.f, 0.f};
   if (wave == 0 && c.correction)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       if (lane + 64 * j < c.experts) early_correction[j] = c.correction[lane + 64 * j];
-  float gate_value = 0.f;
-  for (int first = 0; first < outputs; first += ROUTE_BATCH) {
-    float sums[ROUTE_BATCH];
-    const float* rows[ROUTE_BATCH];                 // an output beyond the last reads the last one's row and is dropped
+  for (int first = wave; first < outputs; first += ROUTE_WAVES * ROUTE_OUTPUTS) {
+    float sums[ROUTE_OUTPUTS];
+    const float* rows[ROUTE_OUTPUTS];               // an output beyond the last reads the last one's row and is dropped
 #pragma unroll
-    for (int j = 0; j < ROUTE_BATCH; ++j) {
+    for (int j = 0; j < ROUTE_OUTPUTS; ++j) {
       sums[j] = 0.f;
-      const int e = first + j < outputs ? first + j : outputs - 1;
+      const int e = first + ROUTE_WAVES * j < outputs ? first + ROUTE_WAVES * j : outputs - 1;
       rows[j] = e < c.experts ? c.W + (int64_t)e * c.width : c.gate_w;
     }
-    // four columns a thread and turn, none of the loads behind a branch of its own: all of a turn's
-    // loads are in flight together (behind branches they are waited for one by one)
-    for (int col0 = threadIdx.x; col0 < c.width; col0 += 4 * ROUTE_THREADS) {
-      int cc[4];
-      float xs[4];
+    for (int col0 = lane; col0 < c.width; col0 += 64 * ROUTE_COLUMNS) {
+      int cc[ROUTE_COLUMNS];
+      float xs[ROUTE_COLUMNS];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int col = col0 + u * ROUTE_THREADS;
+      for (int u = 0; u < ROUTE_COLUMNS; ++u) {
+        const int col = col0 + 64 * u;
         cc[u] = col < c.width ? col : 0;
         xs[u] = to_float(h[cc[u]]);
       }
-      float ws[ROUTE_BATCH][4];
+      float ws[ROUTE_OUTPUTS][ROUTE_COLUMNS];
 #pragma unroll
-      for (int j = 0; j < ROUTE_BATCH; ++j)
+      for (int j = 0; j < ROUTE_OUTPUTS; ++j)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) ws[j][u] = rows[j][cc[u]];
+        for (int u = 0; u < ROUTE_COLUMNS; ++u) ws[j][u] = rows[j][cc[u]];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) xs[u] = col0 + u * ROUTE_THREADS < c.width ? xs[u] : 0.f;
+      for (int u = 0; u < ROUTE_COLUMNS; ++u) xs[u] = col0 + 64 * u < c.width ? xs[u] : 0.f;
 #pragma unroll
-      for (int j = 0; j < ROUTE_BATCH; ++j)
+      for (int j = 0; j < ROUTE_OUTPUTS; ++j)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) sums[j] = fmaf(ws[j][u], xs[u], sums[j]);
+        for (int u = 0; u < ROUTE_COLUMNS; ++u) sums[j] = fmaf(ws[j][u], xs[u], sums[j]);
     }
 #pragma unroll
-    for (int j = 0; j < ROUTE_BATCH; ++j) {
+    for (int j = 0; j < ROUTE_OUTPUTS; ++j) {
       const float sum = wave_sum(sums[j]);
-      if (lane == 0) partial[wave][j] = sum;
+      const int e = first + ROUTE_WAVES * j;
+      if (lane == 0 && e < outputs) {
+        if (e < c.experts) score[e] = sum;
+        else gate_sum = sum;                         // (stored at the end: nothing waits for a store meanwhile)
+      }
     }
-    __syncthreads();
-    if (threadIdx.x < ROUTE_BATCH && first + (int)threadIdx.x < outputs) {
-      float sum = 0.f;
-      for (int w = 0; w < ROUTE_THREADS / 64; ++w) sum += partial[w][threadIdx.x];
-      const int e = first + threadIdx.x;
-      if (e < c.experts) score[e] = sum;
-      else gate_value = sum;                       // (stored at the end: nothing waits for a store meanwhile)
-    }
-    __syncthreads();
   }
+  __syncthreads();
   if (wave != 0) return;
-  if (c.gate_w && (int)threadIdx.x == (outputs - 1) % ROUTE_BATCH) c.gate[t] = 1.0f / (1.0f + expf(-gate_value));
   float top_logit = -INFINITY;
   for (int e = lane; e < c.experts; e += 64) top_logit = fmaxf(top_logit, score[e]);
   top_logit = wave_max(top_logit);
@@ -169,6 +166,7 @@ __global__ void __launch_bounds__(ROUTE_THREADS) route_kernel(RouteCall c) {
   // the one store of a lane's experts: the chosen ones' scores over their sum, zero elsewhere
   const float inverse = 1.0f / (sum + 1e-20f);
   for (int e = lane; e < c.experts; e += 64) weights[e] = choice[e] == INFINITY ? score[e] * inverse : 0.f;
+  if (c.gate_w && lane == 0) c.gate[t] = 1.0f / (1.0f + expf(-gate_sum));
 }
 
 BT_EXPORT int bt_route_call(void* stream, const RouteCall* c) {
